@@ -35,6 +35,8 @@ def architecture_name(raw: Dict[str, Any]) -> str:
     """The reference insists on exactly one entry in `architectures`
     (/root/reference/src/core/engine.rs:166-169)."""
     archs = raw.get("architectures")
+    if archs is None and isinstance(raw.get("architecture"), str):       # families that name themselves in one string
+        return raw["architecture"]
     if not isinstance(archs, list) or len(archs) != 1 or not isinstance(archs[0], str):
         raise ConfigError(
             f"config.json must name exactly one architecture in 'architectures', got {archs!r}")

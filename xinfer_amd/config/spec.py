@@ -37,7 +37,7 @@ class LayerSpec:
     prefix: str
     block: str
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: Optional[PartSpec]      # None: the layer has no feed-forward (block arrangements that allow it)
     norms: Mapping[str, PartSpec]
     mixer_name: str = "self_attn"
     feed_forward_name: str = "mlp"

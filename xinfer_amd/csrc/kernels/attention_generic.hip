@@ -3,7 +3,12 @@
 // the attention of the 32-bit path; the bfloat16 path uses it where no faster kernel
 // applies.  Keys of a token at position p are the cached positions lo..p of its own
 // request, lo = max(0, p - window + 1), read through the request's block table.  K is
-// [page, kv_head, offset, d]; V is the same or, with v_grouped, [page, kv_head, offset / 8, d, 8].
+// [page, kv_head, offset, d]; V is [page, kv_head, offset, dv] or, with v_grouped,
+// [page, kv_head, offset / 8, dv, 8]; the value head size dv may differ from d.
+//
+// Options of the score, each off unless given:  s = (q . k) * scale;  with a soft cap c,
+// s = c * tanh(s / c);  with per-head slopes a[h], s -= a[h] * (p - p') (a bias that grows
+// with the distance to the key).
 //
 // Reference: PagedAttention::forward at /root/reference/src/models/layers/attention.rs:947-958
 // (external kernel); golden formula tests/probes/compare_flashinfer_probe.py:51-73:
@@ -25,7 +30,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tok_seq,
     const int* __restrict__ positions, T* __restrict__ out, float scale, int window, int page_size,
-    int nq, int nkv, int d, int v_grouped) {
+    int nq, int nkv, int d, int dv, int v_grouped, float softcap, const float* __restrict__ slopes) {
   __shared__ float q_s[kMaxHeadDim];
   __shared__ float acc_s[kAttnWaves][kMaxHeadDim];
   __shared__ float m_s[kAttnWaves], l_s[kAttnWaves];
@@ -41,8 +46,10 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
   const int* bt = block_tables + (size_t)seq * max_pages;
 
   const T* qp = q + ((size_t)t * nq + h) * d;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) q_s[i] = to_float(qp[i]) * scale;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) q_s[i] = to_float(qp[i]);
   __syncthreads();
+  const float slope = slopes ? slopes[h] : 0.f;
+  const float inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
 
   constexpr int NE = kMaxHeadDim / kWave;  // output dims per lane
   float acc[NE];
@@ -61,12 +68,14 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
     if (valid) {
       const int page = bt[key / page_size];
       row = (page * nkv + kvh) * page_size + key % page_size;
-      vrow = (page * nkv + kvh) * d;
+      vrow = (page * nkv + kvh) * dv;
       voff = key % page_size;
       const T* kp = k_cache + (size_t)row * d;
       float dot = 0.f;
       for (int i = 0; i < d; ++i) dot = fmaf(q_s[i], to_float(kp[i]), dot);
-      s = dot;
+      s = dot * scale;
+      if (softcap > 0.f) s = softcap * tanhf(s * inv_cap);
+      if (slopes) s -= slope * (float)(pos - key);
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -81,12 +90,12 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
       const int rj = __shfl(row, j, kWave);
       const int vrj = __shfl(vrow, j, kWave);
       const int voj = __shfl(voff, j, kWave);
-      const T* vp = v_cache + (size_t)rj * d;
-      const T* vtp = v_cache + (size_t)vrj * page_size + (size_t)(voj >> 3) * d * 8 + (voj & 7);  // [offset / 8, d, 8] block
+      const T* vp = v_cache + (size_t)rj * dv;
+      const T* vtp = v_cache + (size_t)vrj * page_size + (size_t)(voj >> 3) * dv * 8 + (voj & 7);  // [offset / 8, dv, 8] block
 #pragma unroll
       for (int e = 0; e < NE; ++e) {
         const int i = lane + e * kWave;
-        if (i < d) {
+        if (i < dv) {
           const float vv = v_grouped ? to_float(vtp[(size_t)i * 8]) : to_float(vp[i]);
           acc[e] = fmaf(pj, vv, acc[e]);
         }
@@ -100,7 +109,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
 #pragma unroll
   for (int e = 0; e < NE; ++e) {
     const int i = lane + e * kWave;
-    if (i < d) acc_s[wave][i] = acc[e];
+    if (i < dv) acc_s[wave][i] = acc[e];
   }
   __syncthreads();
   float mm = m_s[0];
@@ -113,8 +122,8 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
     f[w] = (m_s[w] == -INFINITY) ? 0.f : expf(m_s[w] - mm);
     ll += l_s[w] * f[w];
   }
-  T* op = out + ((size_t)t * nq + h) * d;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+  T* op = out + ((size_t)t * nq + h) * dv;
+  for (int i = threadIdx.x; i < dv; i += blockDim.x) {
     float o = 0.f;
 #pragma unroll
     for (int w = 0; w < kAttnWaves; ++w) o += acc_s[w][i] * f[w];
@@ -130,11 +139,14 @@ extern "C" int xi_attention_generic(const void* q, const void* k_cache, const vo
                                     int dtype, const int* block_tables, int max_pages,
                                     const int* tok_seq, const int* positions, void* out,
                                     float scale, int window, int page_size, int n_tok, int nq,
-                                    int nkv, int d, int v_grouped, hipStream_t stream) {
+                                    int nkv, int d, int dv, int v_grouped, float softcap, const float* slopes,
+                                    hipStream_t stream) {
   XI_CHECK(n_tok >= 0 && nq > 0 && nkv > 0 && page_size > 0 && max_pages > 0,
            "attention: bad sizes T=%d nq=%d nkv=%d page=%d max_pages=%d", n_tok, nq, nkv, page_size, max_pages);
   XI_CHECK(nq % nkv == 0, "attention: %d query heads are not a multiple of %d kv heads", nq, nkv);
   XI_CHECK(d > 0 && d <= kMaxHeadDim, "attention: head_dim %d is outside 1..%d", d, kMaxHeadDim);
+  XI_CHECK(dv > 0 && dv <= kMaxHeadDim, "attention: value head size %d is outside 1..%d", dv, kMaxHeadDim);
+  XI_CHECK(softcap >= 0.f, "attention: the soft cap must be positive (0: none), got %g", (double)softcap);
   XI_CHECK(nq <= 65535, "attention: too many heads (%d)", nq);
   XI_CHECK(!v_grouped || page_size % 8 == 0, "attention: V in groups of eight keys needs pages of a multiple of 8 tokens, not %d", page_size);
   if (n_tok == 0) return 0;
@@ -142,11 +154,11 @@ extern "C" int xi_attention_generic(const void* q, const void* k_cache, const vo
   if (dtype == kF32)
     attention_generic_kernel<float><<<grid, kAttnWaves * kWave, 0, stream>>>(
         (const float*)q, (const float*)k_cache, (const float*)v_cache, block_tables, max_pages,
-        tok_seq, positions, (float*)out, scale, window, page_size, nq, nkv, d, v_grouped);
+        tok_seq, positions, (float*)out, scale, window, page_size, nq, nkv, d, dv, v_grouped, softcap, slopes);
   else if (dtype == kBF16)
     attention_generic_kernel<bf16><<<grid, kAttnWaves * kWave, 0, stream>>>(
         (const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, block_tables, max_pages,
-        tok_seq, positions, (bf16*)out, scale, window, page_size, nq, nkv, d, v_grouped);
+        tok_seq, positions, (bf16*)out, scale, window, page_size, nq, nkv, d, dv, v_grouped, softcap, slopes);
   else
     XI_CHECK(false, "attention: unknown dtype %d", dtype);
   XI_LAUNCH_CHECK("attention_generic");

@@ -471,6 +471,139 @@ __global__ void lane_xor_probe_kernel(const float* __restrict__ in, float* __res
 
 using namespace xi;
 
+// ---------------------------------------------------------------------------------
+// Embedding with sinusoidal positions added: out[t, c] = float(table[ids[t], c]) * scale + pe(p, c),
+// pe(p, 2i) = sin(p * f[i]), pe(p, 2i + 1) = cos(p * f[i]) with p = positions[t] and f the table of
+// frequencies the host made (base^(-2i / H)); angles, sines and the sum in float32.  `rows`, if given,
+// also gets the sum rounded to the activation type (what the first layer's products read).
+// ---------------------------------------------------------------------------------
+template <typename T, typename TR>
+__global__ void embed_sinusoid_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                                      const int* __restrict__ positions, const float* __restrict__ freq,
+                                      float* __restrict__ out, TR* __restrict__ rows, int H, float scale) {
+  const int t = blockIdx.x;
+  const T* row = table + (size_t)ids[t] * H;
+  const float p = (float)positions[t];
+  float* o = out + (size_t)t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float ang = p * freq[i >> 1];
+    const float pe = (i & 1) ? cosf(ang) : sinf(ang);
+    const float v = to_float(row[i]) * scale + pe;
+    o[i] = v;
+    if (rows) rows[(size_t)t * H + i] = from_float<TR>(v);
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// RMSNorm of a branch's output, added into the residual stream (the arrangement in which a
+// sublayer reads the stream itself and its OUTPUT is normed):
+//   s = y[row] (a stack of `parts` partial sums is added in order);
+//   resid[row] += s * rsqrt(mean(s^2) + eps) * w;   rows[row] = round(resid[row]) if asked for.
+// w == null: no norm, resid += s.  Everything in float32.
+// ---------------------------------------------------------------------------------
+template <typename TY, typename TR, int NT>
+__global__ __launch_bounds__(NT) void rmsnorm_add_kernel(float* __restrict__ resid, const TY* __restrict__ y, int parts,
+                                                         size_t part_stride, const float* __restrict__ w, float eps,
+                                                         TR* __restrict__ rows, int H) {
+  __shared__ float scratch[NT / kWave];
+  const int row = blockIdx.x;
+  float* x = resid + (size_t)row * H;
+  const TY* yr = y + (size_t)row * H;
+  float inv = 1.f;
+  if (w) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += NT) {
+      float s = to_float(yr[i]);
+      for (int p = 1; p < parts; ++p) s += to_float(yr[p * part_stride + i]);
+      ss += s * s;
+    }
+    const float total = block_sum<NT / kWave>(ss, scratch);
+    inv = rsqrtf(total / (float)H + eps);
+  }
+  for (int i = threadIdx.x; i < H; i += NT) {
+    float s = to_float(yr[i]);
+    for (int p = 1; p < parts; ++p) s += to_float(yr[p * part_stride + i]);
+    const float v = x[i] + (w ? s * inv * w[i] : s);
+    x[i] = v;
+    if (rows) rows[(size_t)row * H + i] = from_float<TR>(v);
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// act(gate) * up for a packed [T, 2I] buffer, the activation chosen by code:
+// 0 silu(z) = z * sigmoid(z); 1 the tanh form of gelu, 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
+// ---------------------------------------------------------------------------------
+enum Act : int { kSilu = 0, kGeluTanh = 1 };
+template <int ACT>
+__device__ __forceinline__ float act_of(float z) {
+  if constexpr (ACT == kSilu) return z / (1.f + expf(-z));
+  else return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+template <typename T, int ACT>
+__global__ void act_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / I, i = idx - t * I;
+    const float g = to_float(gu[t * 2 * I + i]), u = to_float(gu[t * 2 * I + I + i]);
+    out[idx] = from_float<T>(act_of<ACT>(g) * u);
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// A packed projection row [q (nq d) | k (nkv d) | v (nkv dv)] made ready for attention without
+// rotation: RMSNorm over the WHOLE q part and the whole k part (one mean over all heads, weights of
+// that length; off if the weights are null), v blended with another layer's values of the same token,
+// v = (1 - mix) v + mix v_other (off if v_other is null), q to q_out [T, nq, d], k and v into the paged
+// cache at `slots` (a negative slot stores nothing).  K pool [pages, nkv, page, d]; V pool
+// [pages, nkv, page, dv] or, grouped, [pages, nkv, page / 8, dv, 8].  Norms and the blend in float32.
+// ---------------------------------------------------------------------------------
+template <typename T, int NT>
+__global__ __launch_bounds__(NT) void qkv_rows_kernel(const T* __restrict__ qkv, const float* __restrict__ qw,
+                                                      const float* __restrict__ kw, float eps,
+                                                      const T* __restrict__ v_other, long long v_other_stride, float mix,
+                                                      const long long* __restrict__ slots, T* __restrict__ q_out,
+                                                      T* __restrict__ k_cache, T* __restrict__ v_cache, int page_size,
+                                                      int nq, int nkv, int d, int dv, int v_grouped) {
+  __shared__ float scratch[NT / kWave];
+  const int t = blockIdx.x;
+  const int nqd = nq * d, nkd = nkv * d, nvd = nkv * dv;
+  const T* row = qkv + (size_t)t * (nqd + nkd + nvd);
+  float invq = 1.f, invk = 1.f;
+  if (qw) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < nqd; i += NT) {
+      const float v = to_float(row[i]);
+      ss += v * v;
+    }
+    invq = rsqrtf(block_sum<NT / kWave>(ss, scratch) / (float)nqd + eps);
+    ss = 0.f;
+    for (int i = threadIdx.x; i < nkd; i += NT) {
+      const float v = to_float(row[nqd + i]);
+      ss += v * v;
+    }
+    invk = rsqrtf(block_sum<NT / kWave>(ss, scratch) / (float)nkd + eps);
+  }
+  for (int i = threadIdx.x; i < nqd; i += NT)
+    q_out[(size_t)t * nqd + i] = from_float<T>(qw ? to_float(row[i]) * invq * qw[i] : to_float(row[i]));
+  const long long slot = slots[t];
+  if (slot < 0) return;
+  const size_t page = (size_t)(slot / page_size);
+  const int off = (int)(slot % page_size);
+  for (int i = threadIdx.x; i < nkd; i += NT) {
+    const int h = i / d, c = i - h * d;
+    const float v = to_float(row[nqd + i]);
+    k_cache[((page * nkv + h) * page_size + off) * d + c] = from_float<T>(kw ? v * invk * kw[i] : v);
+  }
+  const T* vo = v_other ? v_other + (size_t)t * v_other_stride : nullptr;
+  for (int i = threadIdx.x; i < nvd; i += NT) {
+    const int h = i / dv, c = i - h * dv;
+    float v = to_float(row[nqd + nkd + i]);
+    if (vo) v = (1.f - mix) * v + mix * to_float(vo[i]);
+    const size_t base = (page * nkv + h) * (size_t)page_size * dv;
+    const size_t at = v_grouped ? base + ((size_t)(off >> 3) * dv + c) * 8 + (off & 7) : base + (size_t)off * dv + c;
+    v_cache[at] = from_float<T>(v);
+  }
+}
+
 extern "C" {
 
 const char* xi_last_error() { return g_error; }
@@ -627,6 +760,86 @@ int xi_qk_norm_rope_kv(const void* qkv, int dtype, int slices, const float* bias
   else XI_CHECK(false, "qk_norm_rope_kv: unknown dtype %d", dtype);
 #undef XI_QK
   XI_LAUNCH_CHECK("qk_norm_rope_kv");
+  return 0;
+}
+
+// rows: null, or [T, H] in `rows_dtype`.  freq: float32 [(H + 1) / 2].
+int xi_embed_sinusoid(const void* table, int dtype, const int* ids, const int* positions, const float* freq, float* out,
+                      void* rows, int rows_dtype, int n_tok, int H, float scale, hipStream_t stream) {
+  XI_CHECK(n_tok >= 0 && H > 0, "embed_sinusoid: bad sizes T=%d H=%d", n_tok, H);
+  if (n_tok == 0) return 0;
+#define XI_ES(TT, TR) \
+  embed_sinusoid_kernel<TT, TR><<<n_tok, 256, 0, stream>>>((const TT*)table, ids, positions, freq, out, (TR*)rows, H, scale)
+  if (dtype == kF32 && (rows == nullptr || rows_dtype == kF32)) XI_ES(float, float);
+  else if (dtype == kBF16 && (rows == nullptr || rows_dtype == kBF16)) XI_ES(bf16, bf16);
+  else if (dtype == kBF16 && rows_dtype == kF32) XI_ES(bf16, float);
+  else if (dtype == kF32 && rows_dtype == kBF16) XI_ES(float, bf16);
+  else XI_CHECK(false, "embed_sinusoid: unknown dtypes %d %d", dtype, rows_dtype);
+#undef XI_ES
+  XI_LAUNCH_CHECK("embed_sinusoid");
+  return 0;
+}
+
+// y: [T, H] or `parts` partial sums [parts, T, H]; w null: plain add; rows null or [T, H] in rows_dtype.
+int xi_rmsnorm_add(float* resid, const void* y, int y_dtype, int parts, const float* w, float eps, void* rows,
+                   int rows_dtype, int n_rows, int H, hipStream_t stream) {
+  XI_CHECK(n_rows >= 0 && H > 0 && parts >= 1, "rmsnorm_add: bad sizes rows=%d H=%d parts=%d", n_rows, H, parts);
+  if (n_rows == 0) return 0;
+  const size_t part_stride = (size_t)n_rows * H;
+  constexpr int NT = 256;
+#define XI_RA(TY, TR) \
+  rmsnorm_add_kernel<TY, TR, NT><<<n_rows, NT, 0, stream>>>(resid, (const TY*)y, parts, part_stride, w, eps, (TR*)rows, H)
+  if (y_dtype == kF32 && (rows == nullptr || rows_dtype == kF32)) XI_RA(float, float);
+  else if (y_dtype == kF32 && rows_dtype == kBF16) XI_RA(float, bf16);
+  else if (y_dtype == kBF16 && (rows == nullptr || rows_dtype == kBF16)) XI_RA(bf16, bf16);
+  else if (y_dtype == kBF16 && rows_dtype == kF32) XI_RA(bf16, float);
+  else XI_CHECK(false, "rmsnorm_add: unknown dtypes %d %d", y_dtype, rows_dtype);
+#undef XI_RA
+  XI_LAUNCH_CHECK("rmsnorm_add");
+  return 0;
+}
+
+int xi_act_mul(const void* gate_up, void* out, int dtype, int act, int n_tok, int I, hipStream_t stream) {
+  XI_CHECK(n_tok >= 0 && I > 0, "act_mul: bad sizes T=%d I=%d", n_tok, I);
+  XI_CHECK(act == kSilu || act == kGeluTanh, "act_mul: unknown activation %d", act);
+  if (n_tok == 0) return 0;
+  const size_t total = (size_t)n_tok * I;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65535u * 16u) blocks = 65535u * 16u;
+#define XI_AM(TT, A) act_mul_kernel<TT, A><<<(unsigned)blocks, 256, 0, stream>>>((const TT*)gate_up, (TT*)out, I, total)
+  if (dtype == kF32 && act == kSilu) XI_AM(float, kSilu);
+  else if (dtype == kF32) XI_AM(float, kGeluTanh);
+  else if (dtype == kBF16 && act == kSilu) XI_AM(bf16, kSilu);
+  else if (dtype == kBF16) XI_AM(bf16, kGeluTanh);
+  else XI_CHECK(false, "act_mul: unknown dtype %d", dtype);
+#undef XI_AM
+  XI_LAUNCH_CHECK("act_mul");
+  return 0;
+}
+
+// qkv [T, nq d + nkv d + nkv dv]; v_other null or rows of v_other_stride elements holding [nkv dv] values each.
+int xi_qkv_rows(const void* qkv, int dtype, const float* qw, const float* kw, float eps, const void* v_other,
+                long long v_other_stride, float mix, const long long* slots, void* q_out, void* k_cache, void* v_cache,
+                int page_size, int n_tok, int nq, int nkv, int d, int dv, int v_grouped, hipStream_t stream) {
+  XI_CHECK(n_tok >= 0 && nq > 0 && nkv > 0 && d > 0 && dv > 0 && page_size > 0,
+           "qkv_rows: bad sizes T=%d nq=%d nkv=%d d=%d dv=%d page=%d", n_tok, nq, nkv, d, dv, page_size);
+  XI_CHECK((qw == nullptr) == (kw == nullptr), "qkv_rows: q and k norm weights must both be given or both absent");
+  XI_CHECK(!v_grouped || page_size % 8 == 0, "qkv_rows: V in groups of eight keys needs pages of a multiple of 8 tokens, not %d",
+           page_size);
+  XI_CHECK(v_other == nullptr || v_other_stride >= (long long)nkv * dv, "qkv_rows: the other values' rows are too short");
+  if (n_tok == 0) return 0;
+  constexpr int NT = 256;
+  if (dtype == kF32)
+    qkv_rows_kernel<float, NT><<<n_tok, NT, 0, stream>>>((const float*)qkv, qw, kw, eps, (const float*)v_other, v_other_stride,
+                                                         mix, slots, (float*)q_out, (float*)k_cache, (float*)v_cache,
+                                                         page_size, nq, nkv, d, dv, v_grouped);
+  else if (dtype == kBF16)
+    qkv_rows_kernel<bf16, NT><<<n_tok, NT, 0, stream>>>((const bf16*)qkv, qw, kw, eps, (const bf16*)v_other, v_other_stride,
+                                                        mix, slots, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, page_size,
+                                                        nq, nkv, d, dv, v_grouped);
+  else
+    XI_CHECK(false, "qkv_rows: unknown dtype %d", dtype);
+  XI_LAUNCH_CHECK("qkv_rows");
   return 0;
 }
 

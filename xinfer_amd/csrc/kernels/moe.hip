@@ -1,0 +1,218 @@
+// Routed experts (mixture of experts): the router, and the experts' products in a form that
+// serves any sizes and both precisions, one (token, chosen expert) pair at a time.
+//
+//   router   z = Wr x + b in float32 (x may be the activation type's rounding of the stream);
+//            the `top` experts with the largest z (ties: the lower index), their weights the
+//            softmax over the chosen logits only.
+//   expert   y_e = Wd_e (act(Wg_e x) * (Wu_e x)), no biases; gate and up of all experts are stacked
+//            [E, 2F, H] (gate rows first), down [E, H, F].
+//   output   sum over the chosen experts, in the order they were chosen, of weight * y_e: float32.
+//
+// Every sum runs in an order fixed by the sizes alone (lanes stride over k, then the wave's
+// butterfly), so a token's result does not depend on the batch it is in.  The grouped
+// matrix-core products for many tokens are in moe_mfma.hip; this file is the float32 path and
+// what decode steps of few tokens use (a pair reads its expert's weights once: the least traffic
+// there is when every pair has another expert).
+#include "common.h"
+
+namespace xi {
+
+constexpr int kRouteWaves = 4;
+constexpr int kMaxExperts = 1024;
+constexpr int kMaxTop = 64;
+
+template <typename T>
+__global__ __launch_bounds__(kRouteWaves* kWave) void moe_route_kernel(const T* __restrict__ x,
+                                                                       const float* __restrict__ wr,
+                                                                       const float* __restrict__ br, int* __restrict__ idx,
+                                                                       float* __restrict__ wt, int H, int E, int top) {
+  __shared__ float z[kMaxExperts];
+  __shared__ float chosen[kMaxTop];
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const T* xr = x + (size_t)t * H;
+  for (int e = wave; e < E; e += kRouteWaves) {
+    const float* w = wr + (size_t)e * H;
+    float acc = 0.f;
+    for (int k = lane; k < H; k += kWave) acc = fmaf(to_float(xr[k]), w[k], acc);
+    acc = wave_sum(acc);
+    if (lane == 0) z[e] = acc + (br ? br[e] : 0.f);
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  for (int r = 0; r < top; ++r) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < E; e += kWave)
+      if (z[e] > best) {
+        best = z[e];
+        at = e;
+      }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, kWave);
+      const int oa = __shfl_xor(at, o, kWave);
+      if (ob > best || (ob == best && oa < at)) {
+        best = ob;
+        at = oa;
+      }
+    }
+    if (at >= E) at = E - 1;            // no finite logit left (rows of NaN): any valid expert
+    if (lane == 0) {
+      idx[(size_t)t * top + r] = at;
+      chosen[r] = best;
+      z[at] = -INFINITY;
+    }
+    __builtin_amdgcn_s_waitcnt(0);      // lane 0's write to LDS is done before the wave reads z again
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (lane == 0) {
+    const float m = chosen[0];
+    float sum = 0.f;
+    for (int r = 0; r < top; ++r) sum += expf(chosen[r] - m);
+    for (int r = 0; r < top; ++r) wt[(size_t)t * top + r] = expf(chosen[r] - m) / sum;
+  }
+}
+
+template <int ACT>
+__device__ __forceinline__ float moe_act(float z) {
+  if constexpr (ACT == 0) return z / (1.f + expf(-z));
+  else return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// One workgroup: a pair (token, rank) and FT features of its expert; the token's row sits in LDS.
+constexpr int kMoeWaves = 4;
+template <typename T, int ACT>
+__global__ __launch_bounds__(kMoeWaves* kWave) void moe_gate_up_kernel(const T* __restrict__ x, const T* __restrict__ wgu,
+                                                                       const int* __restrict__ idx, T* __restrict__ mid,
+                                                                       int H, int F, int top, int FT) {
+  extern __shared__ float xs[];
+  const int pair = blockIdx.x, t = pair / top;
+  const int e = idx[pair];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  for (int k = threadIdx.x; k < H; k += blockDim.x) xs[k] = to_float(x[(size_t)t * H + k]);
+  __syncthreads();
+  const T* wg = wgu + (size_t)e * 2 * F * H;
+  const int f_end = min(F, (int)(blockIdx.y + 1) * FT);
+  for (int f = blockIdx.y * FT + wave; f < f_end; f += kMoeWaves) {
+    const T* g = wg + (size_t)f * H;
+    const T* u = wg + (size_t)(F + f) * H;
+    float ag = 0.f, au = 0.f;
+    for (int k = lane; k < H; k += kWave) {
+      ag = fmaf(to_float(g[k]), xs[k], ag);
+      au = fmaf(to_float(u[k]), xs[k], au);
+    }
+    ag = wave_sum(ag);
+    au = wave_sum(au);
+    if (lane == 0) mid[(size_t)pair * F + f] = from_float<T>(moe_act<ACT>(ag) * au);
+  }
+}
+
+// One workgroup: a token and NTile output features; the token's `top` rows of mid sit in LDS.
+template <typename T>
+__global__ __launch_bounds__(kMoeWaves* kWave) void moe_down_kernel(const T* __restrict__ mid, const T* __restrict__ wd,
+                                                                    const int* __restrict__ idx, const float* __restrict__ wt,
+                                                                    float* __restrict__ out, int H, int F, int top, int NTile) {
+  extern __shared__ float ms[];       // [top, F]
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  for (int i = threadIdx.x; i < top * F; i += blockDim.x) ms[i] = to_float(mid[(size_t)t * top * F + i]);
+  __syncthreads();
+  const int n_end = min(H, (int)(blockIdx.y + 1) * NTile);
+  for (int n = blockIdx.y * NTile + wave; n < n_end; n += kMoeWaves) {
+    float total = 0.f;
+    for (int r = 0; r < top; ++r) {
+      const T* w = wd + ((size_t)idx[(size_t)t * top + r] * H + n) * F;
+      float acc = 0.f;
+      for (int f = lane; f < F; f += kWave) acc = fmaf(to_float(w[f]), ms[r * F + f], acc);
+      acc = wave_sum(acc);
+      total += wt[(size_t)t * top + r] * acc;
+    }
+    if (lane == 0) out[(size_t)t * H + n] = total;
+  }
+}
+
+}  // namespace xi
+
+using namespace xi;
+
+extern "C" {
+
+// x [T, H] in `dtype`; wr float32 [E, H]; br float32 [E] or null; idx int32 [T, top]; wt float32 [T, top].
+int xi_moe_route(const void* x, int dtype, const float* wr, const float* br, int* idx, float* wt, int n_tok, int H, int E,
+                 int top, hipStream_t stream) {
+  XI_CHECK(n_tok >= 0 && H > 0 && E > 0 && E <= kMaxExperts, "moe_route: bad sizes T=%d H=%d experts=%d (at most %d)", n_tok,
+           H, E, kMaxExperts);
+  XI_CHECK(top > 0 && top <= E && top <= kMaxTop, "moe_route: %d of %d experts cannot be chosen (at most %d)", top, E, kMaxTop);
+  if (n_tok == 0) return 0;
+  if (dtype == kF32)
+    moe_route_kernel<float><<<n_tok, kRouteWaves * kWave, 0, stream>>>((const float*)x, wr, br, idx, wt, H, E, top);
+  else if (dtype == kBF16)
+    moe_route_kernel<bf16><<<n_tok, kRouteWaves * kWave, 0, stream>>>((const bf16*)x, wr, br, idx, wt, H, E, top);
+  else
+    XI_CHECK(false, "moe_route: unknown dtype %d", dtype);
+  XI_LAUNCH_CHECK("moe_route");
+  return 0;
+}
+
+// x [T, H], wgu [E, 2F, H], idx [T * top] -> mid [T * top, F] = act(gate) * up, all in `dtype`.
+int xi_moe_gate_up(const void* x, const void* wgu, const int* idx, void* mid, int dtype, int act, int n_tok, int H, int F,
+                   int E, int top, hipStream_t stream) {
+  XI_CHECK(n_tok >= 0 && H > 0 && F > 0 && E > 0 && top > 0, "moe_gate_up: bad sizes T=%d H=%d F=%d E=%d top=%d", n_tok, H, F, E,
+           top);
+  XI_CHECK(act == 0 || act == 1, "moe_gate_up: unknown activation %d", act);
+  XI_CHECK((size_t)H * sizeof(float) <= 64 * 1024, "moe_gate_up: a row of %d does not fit in LDS", H);
+  if (n_tok == 0) return 0;
+  const long long pairs = (long long)n_tok * top;
+  XI_CHECK(pairs < (1ll << 31), "moe_gate_up: too many tokens");
+  const int FT = 64;
+  dim3 grid((unsigned)pairs, (unsigned)((F + FT - 1) / FT));
+  XI_CHECK(grid.y <= 65535u, "moe_gate_up: F=%d is too large", F);
+  const size_t lds = (size_t)H * sizeof(float);
+#define XI_GU(TT, A)                                                                                            \
+  do {                                                                                                          \
+    auto kern = moe_gate_up_kernel<TT, A>;                                                                      \
+    if (lds > 48 * 1024) {                                                                                      \
+      hipError_t e_ = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+      XI_CHECK(e_ == hipSuccess, "moe_gate_up: cannot get %zu bytes of LDS", lds);                              \
+    }                                                                                                           \
+    kern<<<grid, kMoeWaves * kWave, lds, stream>>>((const TT*)x, (const TT*)wgu, idx, (TT*)mid, H, F, top, FT); \
+  } while (0)
+  if (dtype == kF32 && act == 0) XI_GU(float, 0);
+  else if (dtype == kF32) XI_GU(float, 1);
+  else if (dtype == kBF16 && act == 0) XI_GU(bf16, 0);
+  else if (dtype == kBF16) XI_GU(bf16, 1);
+  else XI_CHECK(false, "moe_gate_up: unknown dtype %d", dtype);
+#undef XI_GU
+  XI_LAUNCH_CHECK("moe_gate_up");
+  return 0;
+}
+
+// mid [T * top, F], wd [E, H, F] in `dtype`; idx, wt [T, top] -> out float32 [T, H].
+int xi_moe_down(const void* mid, const void* wd, const int* idx, const float* wt, float* out, int dtype, int n_tok, int H,
+                int F, int E, int top, hipStream_t stream) {
+  XI_CHECK(n_tok >= 0 && H > 0 && F > 0 && E > 0 && top > 0, "moe_down: bad sizes T=%d H=%d F=%d E=%d top=%d", n_tok, H, F, E, top);
+  const size_t lds = (size_t)top * F * sizeof(float);
+  XI_CHECK(lds <= 64 * 1024, "moe_down: %d rows of %d do not fit in LDS", top, F);
+  if (n_tok == 0) return 0;
+  const int NTile = 64;
+  dim3 grid((unsigned)n_tok, (unsigned)((H + NTile - 1) / NTile));
+  XI_CHECK(grid.y <= 65535u, "moe_down: H=%d is too large", H);
+#define XI_DN(TT)                                                                                               \
+  do {                                                                                                          \
+    auto kern = moe_down_kernel<TT>;                                                                            \
+    if (lds > 48 * 1024) {                                                                                      \
+      hipError_t e_ = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+      XI_CHECK(e_ == hipSuccess, "moe_down: cannot get %zu bytes of LDS", lds);                                 \
+    }                                                                                                           \
+    kern<<<grid, kMoeWaves * kWave, lds, stream>>>((const TT*)mid, (const TT*)wd, idx, wt, out, H, F, top, NTile); \
+  } while (0)
+  if (dtype == kF32) XI_DN(float);
+  else if (dtype == kBF16) XI_DN(bf16);
+  else XI_CHECK(false, "moe_down: unknown dtype %d", dtype);
+#undef XI_DN
+  XI_LAUNCH_CHECK("moe_down");
+  return 0;
+}
+
+}  // extern "C"

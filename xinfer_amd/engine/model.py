@@ -112,7 +112,9 @@ class CausalLM:
                 want_rows: torch.Tensor) -> torch.Tensor:
         """ids int32 [T]; caches: layer index -> the cache that layer owns; want_rows int32
         [R].  Returns float32 logits [R, vocab]."""
-        stream = Stream(self.embedding.forward(ids, ctx), None)
+        first = self.embedding.forward(ids, ctx)
+        # an embedding kind may also hand on its result rounded to the activation dtype (`rows`)
+        stream = Stream(first, None, rows=getattr(self.embedding, "rows", None))
         schedule = self.spec.schedule
         for i, e in enumerate(schedule):
             owner = e.layer if e.cache_of is None else e.cache_of

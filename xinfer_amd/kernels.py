@@ -191,6 +191,157 @@ def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
     return out
 
 
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def act_mul(gate_up: torch.Tensor, act: str = "silu") -> torch.Tensor:
+    """out = act(gate_up[:, :I]) * gate_up[:, I:] for an activation of `ACTIVATIONS` (float32 inside)."""
+    _dev(gate_up)
+    if act not in ACTIVATIONS:
+        raise KernelError(f"act_mul: unknown activation {act!r} ({', '.join(ACTIVATIONS)})")
+    if gate_up.dim() != 2 or gate_up.shape[1] % 2:
+        raise KernelError("act_mul: input must be [T, 2I]")
+    T, I = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((T, I), dtype=gate_up.dtype, device=gate_up.device)
+    _ok(lib().xi_act_mul(_p(gate_up), _p(out), _code(gate_up, "act_mul"), ACTIVATIONS[act], T, I, _stream()))
+    return out
+
+
+def embed_sinusoid(table: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor, freq: torch.Tensor,
+                   scale: float = 1.0, rows_dtype: Optional[torch.dtype] = None):
+    """out[t, c] = float32(table[ids[t], c]) * scale + (sin if c even else cos)(positions[t] * freq[c // 2]).
+    Returns (out float32 [T, H], rows): rows is out rounded to `rows_dtype`, None if not asked for."""
+    _dev(table, ids, positions, freq)
+    _want(ids, torch.int32, "embed_sinusoid: ids")
+    _want(positions, torch.int32, "embed_sinusoid: positions")
+    _want(freq, torch.float32, "embed_sinusoid: freq")
+    if table.dim() != 2 or ids.dim() != 1 or positions.shape != ids.shape:
+        raise KernelError("embed_sinusoid: table must be [V, H], ids and positions [T]")
+    T, H = ids.shape[0], table.shape[1]
+    if freq.shape != ((H + 1) // 2,):
+        raise KernelError(f"embed_sinusoid: {tuple(freq.shape)} frequencies for a width of {H}")
+    out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    rows = None if rows_dtype is None else torch.empty((T, H), dtype=rows_dtype, device=table.device)
+    _ok(lib().xi_embed_sinusoid(_p(table), _code(table, "embed_sinusoid"), _p(ids), _p(positions), _p(freq), _p(out),
+                                _p(rows), _code(rows, "embed_sinusoid") if rows is not None else F32, T, H,
+                                ctypes.c_float(scale), _stream()))
+    return out, rows
+
+
+def rmsnorm_add(resid: torch.Tensor, y: torch.Tensor, weight: Optional[torch.Tensor], eps: float,
+                rows_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """resid += rms(y) * weight in place (float32), y [T, H] or a stack [P, T, H] of partial sums added in
+    order; without `weight` resid += y.  Returns resid rounded to `rows_dtype` ([T, H]) if asked for."""
+    _dev(resid, y, weight)
+    _want(resid, torch.float32, "rmsnorm_add: residual stream")
+    if resid.dim() != 2:
+        raise KernelError("rmsnorm_add: the residual stream must be [T, H]")
+    T, H = resid.shape
+    parts = 1
+    if y.dim() == 3:
+        parts = int(y.shape[0])
+        if tuple(y.shape[1:]) != (T, H) or parts < 1:
+            raise KernelError(f"rmsnorm_add: partial sums {tuple(y.shape)} must be [P, {T}, {H}]")
+    elif tuple(y.shape) != (T, H):
+        raise KernelError(f"rmsnorm_add: y {tuple(y.shape)} differs from resid {(T, H)}")
+    if weight is not None:
+        _want(weight, torch.float32, "rmsnorm_add: weight")
+        if weight.shape != (H,):
+            raise KernelError(f"rmsnorm_add: weight {tuple(weight.shape)} is not [{H}]")
+    rows = None if rows_dtype is None else torch.empty((T, H), dtype=rows_dtype, device=resid.device)
+    _ok(lib().xi_rmsnorm_add(_p(resid), _p(y), _code(y, "rmsnorm_add"), parts, _p(weight), ctypes.c_float(eps), _p(rows),
+                             _code(rows, "rmsnorm_add") if rows is not None else F32, T, H, _stream()))
+    return rows
+
+
+def qkv_rows(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
+             slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, num_heads: int, num_kv_heads: int,
+             head_dim: int, value_dim: int, v_grouped: bool = False, v_other: Optional[torch.Tensor] = None,
+             mix: float = 0.0) -> torch.Tensor:
+    """A packed projection [T, nq d + nkv d + nkv dv] made ready for attention without rotation: RMSNorm
+    over the whole q part and the whole k part (weights float32 [nq d] and [nkv d]; none: no norm), v
+    blended with `v_other` ([T, nkv dv], rows may be a strided view: another layer's values of the same
+    tokens) as (1 - mix) v + mix v_other, k and v into the paged cache at `slots`.  Returns q [T, nq, d]."""
+    _dev(qkv, q_weight, k_weight, slots, k_cache, v_cache)
+    nq, nkv, d, dv = int(num_heads), int(num_kv_heads), int(head_dim), int(value_dim)
+    if qkv.dim() != 2 or qkv.shape[1] != nq * d + nkv * d + nkv * dv:
+        raise KernelError(f"qkv_rows: qkv {tuple(qkv.shape)} is not [T, {nq * d + nkv * d + nkv * dv}]")
+    T = qkv.shape[0]
+    _want(slots, torch.int64, "qkv_rows: slots")
+    if slots.shape != (T,):
+        raise KernelError("qkv_rows: slots must be [T]")
+    for w, n in ((q_weight, nq * d), (k_weight, nkv * d)):
+        if w is not None:
+            _want(w, torch.float32, "qkv_rows: norm weight")
+            if w.shape != (n,):
+                raise KernelError(f"qkv_rows: norm weight {tuple(w.shape)} is not [{n}]")
+    _check_cache(k_cache, v_cache, nkv, d, qkv.dtype, v_grouped, "qkv_rows", dv=dv)
+    stride = 0
+    if v_other is not None:
+        if (not v_other.is_cuda or v_other.device != qkv.device or v_other.dtype != qkv.dtype or v_other.dim() != 2
+                or tuple(v_other.shape) != (T, nkv * dv) or v_other.stride(1) != 1):
+            raise KernelError(f"qkv_rows: the other values {tuple(v_other.shape)} {v_other.dtype} must be [{T}, {nkv * dv}] "
+                              "rows of the projection's type")
+        stride = int(v_other.stride(0))
+    q_out = torch.empty((T, nq, d), dtype=qkv.dtype, device=qkv.device)
+    _ok(lib().xi_qkv_rows(_p(qkv), _code(qkv, "qkv_rows"), _p(q_weight), _p(k_weight), ctypes.c_float(eps), _p(v_other),
+                          ctypes.c_longlong(stride), ctypes.c_float(mix), _p(slots), _p(q_out), _p(k_cache), _p(v_cache),
+                          int(k_cache.shape[2]), T, nq, nkv, d, dv, int(bool(v_grouped)), _stream()))
+    return q_out
+
+
+def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int):
+    """Router of a mixture of experts: z = router @ x + bias in float32 (router float32 [E, H]), the `top`
+    largest (ties: the lower index), weights = softmax over the chosen logits.  Returns
+    (idx int32 [T, top], weights float32 [T, top]), the chosen in descending order of their logits."""
+    _dev(x, router, bias)
+    _want(router, torch.float32, "moe_route: router weight")
+    if x.dim() != 2 or router.dim() != 2 or router.shape[1] != x.shape[1]:
+        raise KernelError(f"moe_route: x {tuple(x.shape)} and the router {tuple(router.shape)} do not match")
+    T, H = x.shape
+    E = router.shape[0]
+    if bias is not None:
+        _want(bias, torch.float32, "moe_route: bias")
+        if bias.shape != (E,):
+            raise KernelError(f"moe_route: bias {tuple(bias.shape)} is not [{E}]")
+    if not (0 < top <= min(E, 64)) or E > 1024:
+        raise KernelError(f"moe_route: {top} of {E} experts (at most 64 of 1024)")
+    idx = torch.empty((T, top), dtype=torch.int32, device=x.device)
+    wt = torch.empty((T, top), dtype=torch.float32, device=x.device)
+    _ok(lib().xi_moe_route(_p(x), _code(x, "moe_route"), _p(router), _p(bias), _p(idx), _p(wt), T, H, E, int(top), _stream()))
+    return idx, wt
+
+
+def moe_experts(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx: torch.Tensor, wt: torch.Tensor,
+                act: str = "silu") -> torch.Tensor:
+    """sum over a token's chosen experts e (in the order of `idx`) of wt * down[e] @ (act(gate[e] @ x) * (up[e] @ x)):
+    gate_up [E, 2F, H] (gate rows first), down [E, H, F], idx int32 / wt float32 [T, top].  Float32 [T, H].
+    One (token, expert) pair at a time, every sum in an order fixed by the sizes: the form of the
+    float32 path and of steps with few tokens."""
+    _dev(x, gate_up, down, idx, wt)
+    if act not in ACTIVATIONS:
+        raise KernelError(f"moe_experts: unknown activation {act!r}")
+    if gate_up.dim() != 3 or down.dim() != 3 or x.dim() != 2:
+        raise KernelError("moe_experts: x [T, H], gate_up [E, 2F, H], down [E, H, F]")
+    T, H = x.shape
+    E, F2, _ = gate_up.shape
+    F = F2 // 2
+    if gate_up.shape != (E, 2 * F, H) or down.shape != (E, H, F) or x.dtype != gate_up.dtype or x.dtype != down.dtype:
+        raise KernelError(f"moe_experts: x {tuple(x.shape)} {x.dtype}, gate_up {tuple(gate_up.shape)} {gate_up.dtype} and "
+                          f"down {tuple(down.shape)} {down.dtype} do not match")
+    _want(idx, torch.int32, "moe_experts: idx")
+    _want(wt, torch.float32, "moe_experts: weights")
+    if idx.dim() != 2 or idx.shape[0] != T or wt.shape != idx.shape:
+        raise KernelError("moe_experts: idx and weights must be [T, top]")
+    top = int(idx.shape[1])
+    mid = torch.empty((T * top, F), dtype=x.dtype, device=x.device)
+    out = torch.empty((T, H), dtype=torch.float32, device=x.device)
+    code = _code(x, "moe_experts")
+    _ok(lib().xi_moe_gate_up(_p(x), _p(gate_up), _p(idx), _p(mid), code, ACTIVATIONS[act], T, H, F, E, top, _stream()))
+    _ok(lib().xi_moe_down(_p(mid), _p(down), _p(idx), _p(wt), _p(out), code, T, H, F, E, top, _stream()))
+    return out
+
+
 def qk_norm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
                     k_weight: Optional[torch.Tensor], eps: float, cos: torch.Tensor,
                     sin: torch.Tensor, rotary_dim: int, interleaved: bool,
@@ -247,15 +398,17 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
     return q_out
 
 
-def _check_cache(k_cache, v_cache, nkv, d, dtype, v_grouped, what):
-    """K pool [pages, nkv, page, d]; V pool the same, or [pages, nkv, page / 8, d, 8] if in groups of eight keys."""
+def _check_cache(k_cache, v_cache, nkv, d, dtype, v_grouped, what, dv=None):
+    """K pool [pages, nkv, page, d]; V pool [pages, nkv, page, dv], or [pages, nkv, page / 8, dv, 8] if in
+    groups of eight keys (dv: the value head size, d unless given)."""
+    dv = d if dv is None else int(dv)
     if k_cache.dim() != 4 or k_cache.shape[1] != nkv or k_cache.shape[3] != d or k_cache.dtype != dtype:
         raise KernelError(f"{what}: K pool {tuple(k_cache.shape)} {k_cache.dtype} does not match "
                           f"[pages, {nkv}, page_size, {d}] {dtype}")
     pages, _, page, _ = k_cache.shape
     if v_grouped and page % 8:
         raise KernelError(f"{what}: V in groups of eight keys needs pages of a multiple of 8 tokens, not {page}")
-    want = (pages, nkv, page // 8, d, 8) if v_grouped else (pages, nkv, page, d)
+    want = (pages, nkv, page // 8, dv, 8) if v_grouped else (pages, nkv, page, dv)
     if tuple(v_cache.shape) != want or v_cache.dtype != dtype:
         raise KernelError(f"{what}: V pool {tuple(v_cache.shape)} {v_cache.dtype} does not match {want} {dtype}")
 
@@ -263,31 +416,42 @@ def _check_cache(k_cache, v_cache, nkv, d, dtype, v_grouped, what):
 def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_tables: torch.Tensor, tok_seq: torch.Tensor, positions: torch.Tensor,
                       scale: float, window: int = 0, out: Optional[torch.Tensor] = None,
-                      v_grouped: bool = False) -> torch.Tensor:
+                      v_grouped: bool = False, softcap: float = 0.0,
+                      slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal paged GQA attention for any mix of tokens.  q [T, nq, d]; caches
-    [pages, nkv, page_size, d]; block_tables int32 [B, max_pages]; tok_seq / positions
+    [pages, nkv, page_size, d] (the V pool's last size, the value head size, may differ);
+    block_tables int32 [B, max_pages]; tok_seq / positions
     int32 [T] name each token's row of block_tables and its absolute position.
-    window = 0 keeps all keys, w > 0 the last w (the query's own key included)."""
-    _dev(q, k_cache, v_cache, block_tables, tok_seq, positions, out)
+    window = 0 keeps all keys, w > 0 the last w (the query's own key included).
+    `softcap` c > 0: scores become c * tanh(score / c); `slopes` float32 [nq]: head h's scores lose
+    slopes[h] * (distance from the query to the key)."""
+    _dev(q, k_cache, v_cache, block_tables, tok_seq, positions, out, slopes)
     if q.dim() != 3:
         raise KernelError("attention: q must be [T, nq, d]")
     T, nq, d = q.shape
     if k_cache.dim() != 4:
         raise KernelError("attention: the K pool must be [pages, nkv, page_size, d]")
     nkv, page = k_cache.shape[1], k_cache.shape[2]
-    _check_cache(k_cache, v_cache, nkv, d, q.dtype, v_grouped, "attention")
+    dv = int(v_cache.shape[3])
+    _check_cache(k_cache, v_cache, nkv, d, q.dtype, v_grouped, "attention", dv=dv)
     for t, name in ((block_tables, "block_tables"), (tok_seq, "tok_seq"), (positions, "positions")):
         _want(t, torch.int32, f"attention: {name}")
     if block_tables.dim() != 2 or tok_seq.shape != (T,) or positions.shape != (T,):
         raise KernelError("attention: block_tables must be [B, max_pages], tok_seq and positions [T]")
+    if slopes is not None:
+        _want(slopes, torch.float32, "attention: slopes")
+        if slopes.shape != (nq,):
+            raise KernelError(f"attention: slopes {tuple(slopes.shape)} must be one a query head, [{nq}]")
+    if not softcap >= 0:
+        raise KernelError(f"attention: the soft cap must be positive (0: none), got {softcap}")
     if out is None:
-        out = torch.empty((T, nq * d), dtype=q.dtype, device=q.device)
-    elif out.shape != (T, nq * d) or out.dtype != q.dtype:
+        out = torch.empty((T, nq * dv), dtype=q.dtype, device=q.device)
+    elif out.shape != (T, nq * dv) or out.dtype != q.dtype:
         raise KernelError("attention: out has the wrong shape or dtype")
     _ok(lib().xi_attention_generic(
         _p(q), _p(k_cache), _p(v_cache), _code(q, "attention"), _p(block_tables),
         int(block_tables.shape[1]), _p(tok_seq), _p(positions), _p(out), ctypes.c_float(scale),
-        int(window), int(page), T, nq, nkv, d, int(bool(v_grouped)), _stream()))
+        int(window), int(page), T, nq, nkv, d, dv, int(bool(v_grouped)), ctypes.c_float(softcap), _p(slopes), _stream()))
     return out
 
 
@@ -562,14 +726,20 @@ def attention_decode_packed_bf16(qkv, q_weight, k_weight, eps, cos, sin, rotary_
 
 
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, group: int,
-              scale: float, window: int = 0, v_grouped: bool = False) -> torch.Tensor:
+              scale: float, window: int = 0, v_grouped: bool = False, softcap: float = 0.0,
+              slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of one step's tokens over the paged cache of `group`; chooses the kernel
     from the precision and the shape of the batch: float32, or sizes the matrix-core
     kernels do not take, go to the generic kernel; bfloat16 batches of single tokens to
-    the split-K decode kernel; everything else to the prefill kernel."""
+    the split-K decode kernel; everything else to the prefill kernel.  Scores with a soft cap
+    or a distance bias, and values of another head size than the keys, have matrix-core
+    kernels of their own (`attention_biased_bf16`)."""
     T, nq, d = q.shape
     nkv, page = k_cache.shape[1], k_cache.shape[2]
     bt = ctx.block_tables[group]
+    if softcap > 0 or slopes is not None or v_cache.shape[3] != d:
+        return attention_generic(q, k_cache, v_cache, bt, ctx.tok_seq, ctx.positions, scale, window,
+                                 v_grouped=v_grouped, softcap=softcap, slopes=slopes)
     if q.dtype == torch.bfloat16 and v_grouped and mfma_attention_supported(nq, nkv, d, page):
         g = nq // nkv
         if ctx.max_q_len == 1 and decode_attention_takes(nq, nkv, d):

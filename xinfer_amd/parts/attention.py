@@ -6,6 +6,16 @@ last `window`) -> output projection.  Reference: Attention::forward_with_kv,
 /root/reference/src/models/layers/attention.rs:796-977 (projection 805-828, q/k norm
 709-748, RoPE 872-879, paged attention 947-958, o_proj 976); q, k, v weights are
 concatenated at load as in attention.rs:376-407.
+
+Beside that form the mixer takes, each as a parameter of its spec: values of another head size
+than the keys (`value_dim`); the q/k RMSNorm over the whole projection instead of head by head
+(`qk_norm="row"`, weights as long as the projection); a soft cap c on the scores, c tanh(s / c)
+(`score_softcap`); a bias that takes `distance_slopes[h] * (i - j)` off head h's score of query i
+and key j; values blended with those another layer made for the same token, (1 - m) v + m v_other
+(`value_mix`: the layers of one `key` share the values of the one that is their `source`, m is a
+scalar tensor of the layer); other tensor names (`names`).  Any of these takes the step through
+`_forward_general`: one kernel norms the projection, blends the values and writes the cache, and
+the attention kernels that know the score's options follow.
 """
 from __future__ import annotations
 
@@ -37,13 +47,35 @@ class PagedAttention(Mixer):
         self.qk_norm_eps = float(spec.get("qk_norm_eps", 1e-6))
         self.window = int(spec.get("window") or 0)
         self.scale = float(spec.get("scale", self.d ** -0.5))
+        self.dv = int(spec.get("value_dim") or self.d)
+        self.row_norm = spec.get("qk_norm") == "row"
+        self.softcap = float(spec.get("score_softcap") or 0.0)
+        slopes = spec.get("distance_slopes")
+        self.slope_values = None if slopes is None else tuple(float(a) for a in slopes)
+        if self.slope_values is not None and len(self.slope_values) != self.nq:
+            raise ValueError(f"{len(self.slope_values)} distance slopes for {self.nq} query heads")
+        vm = spec.get("value_mix")
+        self.value_mix_key = None if not vm else str(vm.get("key", "values"))
+        self.value_mix_source = bool(vm and vm.get("source", False))
+        self.mix = 0.0               # the blend's scalar, read at load
+        self.slopes = None           # float32 [nq] on the device
+        # the options that the fused q/k kernel and the attention kernels of the plain form do not know
+        self.general = bool(self.dv != self.d or self.row_norm or self.softcap > 0 or self.slope_values is not None
+                            or self.value_mix_key is not None)
+        if self.general and spec.get("position") is not None:
+            raise NotImplementedError("attention with a soft cap, a distance bias, a row norm, blended values or another "
+                                      "value size takes no rotation (position encoding) yet")
+        if self.general and (self.qk_norm and not self.row_norm or self.bias):
+            raise NotImplementedError("attention with a soft cap, a distance bias, blended values or another value size "
+                                      "takes the q/k norm over the whole projection or none, and no biases")
         if self.nq % self.nkv:
             raise ValueError(f"{self.nq} query heads are not a multiple of {self.nkv} kv heads")
         # A step of single tokens reads nothing on the host where the split-K decode kernel or the
         # generic kernel serves it; sizes that only the prefill kernel takes (more than 16 query heads
         # per kv head) need the step's lengths on the host to lay out its tiles.
-        self.graph_safe = dtype != torch.bfloat16 or kernels.decode_attention_takes(self.nq, self.nkv, self.d)
-        self.decode_packed = (self.DECODE_PACKED and dtype == torch.bfloat16
+        self.graph_safe = (dtype != torch.bfloat16 or kernels.decode_attention_takes(self.nq, self.nkv, self.d)
+                           or self.general)
+        self.decode_packed = (self.DECODE_PACKED and dtype == torch.bfloat16 and not self.general
                               and kernels.decode_attention_takes(self.nq, self.nkv, self.d))
         pos = spec.get("position")
         self.position = position_encoding_class(pos.kind)(pos, dtype) if pos is not None else None
@@ -53,42 +85,62 @@ class PagedAttention(Mixer):
         self.qkv_bias = None         # float32 [(nq + 2 nkv) d], added by the kernel after the projection
 
     # ---- weights -----------------------------------------------------------
+    NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+             "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias",
+             "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "value_mix": "value_mix"}
+
+    @classmethod
+    def _names(cls, spec: PartSpec, prefix: str):
+        """The tensors' names: the spec's `names` (what follows the prefix) over the defaults."""
+        given = spec.get("names") or {}
+        return {k: f"{prefix}.{given.get(k, v)}" for k, v in cls.NAMES.items()}
+
     @classmethod
     def declare(cls, spec: PartSpec, prefix: str) -> List[TensorDecl]:
         h, nq, nkv, d = (int(spec[k]) for k in ("hidden_size", "num_heads", "num_kv_heads", "head_dim"))
-        out = [TensorDecl(f"{prefix}.q_proj.weight", (nq * d, h)),
-               TensorDecl(f"{prefix}.k_proj.weight", (nkv * d, h)),
-               TensorDecl(f"{prefix}.v_proj.weight", (nkv * d, h)),
-               TensorDecl(f"{prefix}.o_proj.weight", (h, nq * d))]
+        dv = int(spec.get("value_dim") or d)
+        n = cls._names(spec, prefix)
+        out = [TensorDecl(n["q"], (nq * d, h)), TensorDecl(n["k"], (nkv * d, h)),
+               TensorDecl(n["v"], (nkv * dv, h)), TensorDecl(n["o"], (h, nq * dv))]
         if spec.get("bias", False):    # q, k and v only: the reference's o_proj has none (attention.rs:596-608)
-            out += [TensorDecl(f"{prefix}.q_proj.bias", (nq * d,)), TensorDecl(f"{prefix}.k_proj.bias", (nkv * d,)),
-                    TensorDecl(f"{prefix}.v_proj.bias", (nkv * d,))]
-        if spec.get("qk_norm", False):
-            out += [TensorDecl(f"{prefix}.q_norm.weight", (d,), "norm"),
-                    TensorDecl(f"{prefix}.k_norm.weight", (d,), "norm")]
+            out += [TensorDecl(n["q_bias"], (nq * d,)), TensorDecl(n["k_bias"], (nkv * d,)),
+                    TensorDecl(n["v_bias"], (nkv * dv,))]
+        if spec.get("qk_norm") == "row":
+            out += [TensorDecl(n["q_norm"], (nq * d,), "norm"), TensorDecl(n["k_norm"], (nkv * d,), "norm")]
+        elif spec.get("qk_norm", False):
+            out += [TensorDecl(n["q_norm"], (d,), "norm"), TensorDecl(n["k_norm"], (d,), "norm")]
+        vm = spec.get("value_mix")
+        if vm and not vm.get("source", False):
+            out.append(TensorDecl(n["value_mix"], (), "mix"))
         return out
 
     def load(self, store: WeightStore, prefix: str, device) -> None:
         def lin(name):
             t = store.get(name, None, device)
             return t.to(self.dtype) if (self.dtype == torch.float32 or t.dtype != torch.float32) else t
-        parts = [lin(f"{prefix}.{n}_proj.weight") for n in ("q", "k", "v")]
+        names = self._names(self.spec, prefix)
+        parts = [lin(names[n]) for n in ("q", "k", "v")]
         common = torch.float32 if any(p.dtype == torch.float32 for p in parts) else parts[0].dtype
         self.qkv = Linear(torch.cat([p.to(common) for p in parts], dim=0))
-        self.o = Linear(lin(f"{prefix}.o_proj.weight"))
+        self.o = Linear(lin(names["o"]))
         if self.bias:
-            self.qkv_bias = torch.cat([store.get(f"{prefix}.{n}_proj.bias", torch.float32, device)
+            self.qkv_bias = torch.cat([store.get(names[f"{n}_bias"], torch.float32, device)
                                        for n in ("q", "k", "v")]).contiguous()
         if self.qk_norm:
-            self.q_norm_w = store.get(f"{prefix}.q_norm.weight", torch.float32, device).contiguous()
-            self.k_norm_w = store.get(f"{prefix}.k_norm.weight", torch.float32, device).contiguous()
+            self.q_norm_w = store.get(names["q_norm"], torch.float32, device).contiguous()
+            self.k_norm_w = store.get(names["k_norm"], torch.float32, device).contiguous()
+        if self.value_mix_key is not None and not self.value_mix_source:
+            self.mix = float(store.get(names["value_mix"], torch.float32, "cpu").reshape(-1)[0])
+        if self.slope_values is not None:
+            self.slopes = torch.tensor(self.slope_values, dtype=torch.float32, device=device)
         if self.position is not None:
             self.position.load(store, prefix, device)
 
     # ---- cache ---------------------------------------------------------------
     def cache_need(self) -> KVNeed:
         # the matrix-core kernels of the bfloat16 path read V in groups of eight keys
-        return KVNeed.keys_values(self.nkv, self.d, self.window, v_grouped=self.dtype == torch.bfloat16)
+        return KVNeed.keys_values(self.nkv, self.d, self.window, v_grouped=self.dtype == torch.bfloat16,
+                                  value_dim=self.dv)
 
     # ---- step ----------------------------------------------------------------
     takes_sink = True
@@ -96,6 +148,8 @@ class PagedAttention(Mixer):
 
     def forward(self, x, ctx: StepContext, cache: LayerCache, sink=None):
         """`x`: rows or a `Folded`; `sink`: see `Part.takes_sink`."""
+        if self.general:
+            return self._forward_general(x, ctx, cache, sink)
         # a decode step of 17 to 256 rows: the tiled split-K product is ahead of the library, and the
         # kernel below adds its partial sums (which the form for prompt portions does not take)
         rows = None if isinstance(x, Folded) else x.shape[0]
@@ -129,3 +183,23 @@ class PagedAttention(Mixer):
             vector_min_tokens=128 if ctx.max_q_len > 1 else self.VECTOR_MIN_DECODE, bias=self.qkv_bias)
         a = kernels.attention(q, cache.k, cache.v, ctx, cache.group, self.scale, self.window, v_grouped=vt)
         return self.o(a, out_dtype=self.dtype, allow_split=True, sink=sink)     # the next norm adds the parts
+
+    def _forward_general(self, x, ctx: StepContext, cache: LayerCache, sink=None):
+        """The step with the options of the module's second paragraph (no rotation)."""
+        qkv = self.qkv(x, out_dtype=self.dtype)
+        slots = ctx.slots[cache.group] if cache.write else ctx.no_slots
+        vt = self.dtype == torch.bfloat16
+        v_other = None
+        if self.value_mix_key is not None:
+            key = ("value_mix", self.value_mix_key)
+            if self.value_mix_source:          # this step's values, as projected, for the layers that blend them in
+                ctx.scratch[key] = qkv[:, (self.nq + self.nkv) * self.d:]
+            else:
+                v_other = ctx.scratch.get(key)
+                if v_other is None:
+                    raise RuntimeError(f"values {self.value_mix_key!r} are blended in before the layer that makes them has run")
+        q = kernels.qkv_rows(qkv, self.q_norm_w, self.k_norm_w, self.qk_norm_eps, slots, cache.k, cache.v,
+                             self.nq, self.nkv, self.d, self.dv, v_grouped=vt, v_other=v_other, mix=self.mix)
+        a = kernels.attention(q, cache.k, cache.v, ctx, cache.group, self.scale, self.window, v_grouped=vt,
+                              softcap=self.softcap, slopes=self.slopes)
+        return self.o(a, out_dtype=self.dtype, allow_split=True, sink=sink)

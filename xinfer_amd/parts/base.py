@@ -14,6 +14,8 @@ runs on the tokens of one step.  A part never learns which model it is in.
                    resid is the float32 residual stream; `add` (if given) is summed into
                    it first; with `rows` only those rows are produced and resid is not
                    changed.
+                   forward_branch(resid, y, rows_dtype): resid += norm(y), for blocks that norm
+                   a sublayer's output instead of its input.
   PositionEncoding data for the mixer's fused kernel (for "rope": cos/sin tables)
   Block            forward(stream, ctx, cache) -> stream, the arrangement of the above
                    around the residual stream.
@@ -71,11 +73,14 @@ class KVNeed:
     pools: Tuple[PoolNeed, ...] = ()
 
     @staticmethod
-    def keys_values(num_kv_heads: int, head_dim: int, window: int = 0, v_grouped: bool = False) -> "KVNeed":
-        """K pool "k" [pages, kv_heads, page_size, head_dim]; V pool "v" the same, or with
-        `v_grouped` [pages, kv_heads, page_size / 8, head_dim, 8] (eight keys side by side for every dim)."""
+    def keys_values(num_kv_heads: int, head_dim: int, window: int = 0, v_grouped: bool = False,
+                    value_dim: Optional[int] = None) -> "KVNeed":
+        """K pool "k" [pages, kv_heads, page_size, head_dim]; V pool "v" [pages, kv_heads, page_size, value_dim]
+        (`value_dim`: head_dim unless given), or with `v_grouped` [pages, kv_heads, page_size / 8, value_dim, 8]
+        (eight keys side by side for every dim)."""
+        dv = head_dim if value_dim is None else int(value_dim)
         k = PoolNeed("k", (num_kv_heads, PAGE, head_dim))
-        v = PoolNeed("v", (num_kv_heads, PAGE_BY_8, head_dim, 8) if v_grouped else (num_kv_heads, PAGE, head_dim))
+        v = PoolNeed("v", (num_kv_heads, PAGE_BY_8, dv, 8) if v_grouped else (num_kv_heads, PAGE, dv))
         return KVNeed(window, (k, v))
 
 
@@ -163,6 +168,8 @@ class Stream:
     resid: torch.Tensor
     pending: Optional[torch.Tensor] = None
     folded: Optional[Folded] = None
+    rows: Optional[torch.Tensor] = None       # `resid` rounded to the activation dtype, as it is now (nothing
+                                              # pending): what a sublayer that reads the stream itself takes
 
 
 class Part:
@@ -211,6 +218,13 @@ class Norm(Part):
     def forward(self, resid: torch.Tensor, add: Optional[torch.Tensor], out_dtype: torch.dtype,
                 rows: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         raise NotImplementedError
+
+    def forward_branch(self, resid: torch.Tensor, y: torch.Tensor, rows_dtype: Optional[torch.dtype]) -> Optional[torch.Tensor]:
+        """The norm of a branch's OUTPUT, added into the stream: resid += norm(y) in place (y rows, or a
+        stack [P, T, H] of float32 partial sums); returns the new resid rounded to `rows_dtype` (None: nothing).
+        For arrangements whose sublayers read the stream itself ("branchnorm"); a norm kind that is only
+        ever used before a sublayer need not have it."""
+        raise NotImplementedError(f"norm kind {getattr(self, 'kind', type(self).__name__)!r} cannot norm a branch's output")
 
 
 class PositionEncoding(Part):

@@ -5,6 +5,10 @@
 Each residual add is carried out by the norm kernel that follows it: a block hands on
 the stream with its feed-forward output still pending, and the next block's first
 norm (or the model's final norm) adds it.
+
+"branchnorm": x <- x + norm1(mixer(x)); x <- x + norm2(ff(x)): the sublayers read the stream
+itself and their OUTPUT is normed; a layer may have no feed-forward.  The norm, the add and
+the rounding of the new stream for the next sublayer are one kernel (`Norm.forward_branch`).
 """
 from __future__ import annotations
 
@@ -12,6 +16,7 @@ from typing import List, Optional
 
 import torch
 
+from .. import kernels
 from ..config.spec import LayerSpec
 from ..weights.store import TensorDecl, WeightStore
 from .base import (Block, Folded, KVNeed, LayerCache, NormSink, StateNeed, StepContext, Stream,
@@ -84,3 +89,65 @@ class PreNormBlock(Block):
         if isinstance(m, Folded):
             return Stream(stream.resid, None, m)
         return Stream(stream.resid, m)
+
+
+@register_block("branchnorm")
+class BranchNormBlock(Block):
+    """`layer.norms` names the norm of the mixer's output first, then the one of the feed-forward's
+    output (absent if the layer has no feed-forward)."""
+
+    def __init__(self, layer: LayerSpec, dtype: torch.dtype):
+        super().__init__(layer, dtype)
+        self.mixer = mixer_class(layer.mixer.kind)(layer.mixer, dtype)
+        self.ffn = (feed_forward_class(layer.feed_forward.kind)(layer.feed_forward, dtype)
+                    if layer.feed_forward is not None else None)
+        items = layer.norm_items(2 if self.ffn is not None else 1)
+        self._names = [n for n, _ in items]
+        self.norms = [norm_class(n.kind)(n, dtype) for _, n in items]
+
+    @classmethod
+    def declare(cls, layer: LayerSpec) -> List[TensorDecl]:
+        p = layer.prefix
+        out = mixer_class(layer.mixer.kind).declare(layer.mixer, f"{p}.{layer.mixer_name}")
+        if layer.feed_forward is not None:
+            out += feed_forward_class(layer.feed_forward.kind).declare(layer.feed_forward, f"{p}.{layer.feed_forward_name}")
+        for name, n in layer.norm_items(2 if layer.feed_forward is not None else 1):
+            out += norm_class(n.kind).declare(n, f"{p}.{name}")
+        return out
+
+    def load(self, store: WeightStore, device) -> None:
+        p = self.layer.prefix
+        self.mixer.load(store, f"{p}.{self.layer.mixer_name}", device)
+        if self.ffn is not None:
+            self.ffn.load(store, f"{p}.{self.layer.feed_forward_name}", device)
+        for name, norm in zip(self._names, self.norms):
+            norm.load(store, f"{p}.{name}", device)
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(p.graph_safe for p in (self.mixer, *self.norms, *(() if self.ffn is None else (self.ffn,))))
+
+    def cache_need(self) -> Optional[KVNeed]:
+        return self.mixer.cache_need()
+
+    def state_need(self) -> Optional[StateNeed]:
+        return self.mixer.state_need()
+
+    def forward(self, stream: Stream, ctx: StepContext, cache: LayerCache) -> Stream:
+        resid = stream.resid
+        if stream.folded is not None:
+            raise RuntimeError("the stream carries a half-done norm of another block")
+        rows_dtype = None if self.dtype == torch.float32 else self.dtype       # float32: the stream is its own rows
+        x = stream.rows
+        if stream.pending is not None:        # a block of another arrangement left its last branch to be added
+            x = kernels.rmsnorm_add(resid, stream.pending, None, 0.0, rows_dtype)
+        if rows_dtype is None:
+            x = resid
+        elif x is None:                       # a stream that came without its rounding (another embedding kind)
+            x = resid.to(self.dtype)
+        a = self.mixer.forward(x, ctx, cache)
+        x = self.norms[0].forward_branch(resid, a, rows_dtype)
+        if self.ffn is not None:
+            m = self.ffn.forward(x if rows_dtype is not None else resid, ctx)
+            x = self.norms[1].forward_branch(resid, m, rows_dtype)
+        return Stream(resid, None, None, rows=x)

@@ -1,7 +1,8 @@
 """Token embedding and the language-model head, as kinds of their own registries.
 
 "embedding": x = E[ids] (times `scale` if the spec gives one; Qwen3 gives none) into the
-float32 residual stream (reference: /root/reference/src/models/qwen3.rs:211-220,302-309).
+float32 residual stream; with `sinusoid_base` b a sinusoidal position vector is added, entry 2i =
+sin(p b^(-2i / dim)), entry 2i + 1 = cos of the same angle, for the token's position p (float32) (reference: /root/reference/src/models/qwen3.rs:211-220,302-309).
 "lm_head": logits = h @ W^T in float32; W is the embedding table when the spec says `tied`
 (qwen3.rs:267-287,367-373); `softcap` c, if the spec gives one, makes them c * tanh(logits / c).
 """
@@ -27,6 +28,9 @@ class Embedding(TokenEmbedding):
         self.vocab = int(spec["vocab_size"])
         self.dim = int(spec["dim"])
         self.scale = float(spec.get("scale") or 1.0)
+        self.sinusoid_base = float(spec.get("sinusoid_base") or 0.0)
+        self.freq: Optional[torch.Tensor] = None      # float32 [(dim + 1) / 2]: base^(-2i / dim)
+        self.rows: Optional[torch.Tensor] = None      # the last step's result rounded to the activation dtype
         self.table: Optional[torch.Tensor] = None
 
     @classmethod
@@ -38,9 +42,18 @@ class Embedding(TokenEmbedding):
         if self.dtype == torch.float32 or t.dtype != torch.float32:
             t = t.to(self.dtype)
         self.table = t.contiguous()
+        if self.sinusoid_base > 0:
+            i = torch.arange((self.dim + 1) // 2, dtype=torch.float32)
+            self.freq = (torch.tensor(self.sinusoid_base, dtype=torch.float32) ** (-2.0 * i / self.dim)).to(device).contiguous()
 
     def forward(self, ids: torch.Tensor, ctx: Optional[StepContext] = None) -> torch.Tensor:
-        return kernels.embed(self.table, ids, scale=self.scale)
+        if self.freq is None:
+            return kernels.embed(self.table, ids, scale=self.scale)
+        if ctx is None:
+            raise ValueError("an embedding with sinusoidal positions needs the step's positions")
+        out, self.rows = kernels.embed_sinusoid(self.table, ids, ctx.positions, self.freq, self.scale,
+                                                None if self.dtype == torch.float32 else self.dtype)
+        return out
 
 
 @register_head("lm_head")

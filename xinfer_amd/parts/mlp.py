@@ -1,4 +1,4 @@
-"""Gated feed-forward (SwiGLU): down(silu(gate(x)) * up(x)).
+"""Gated feed-forward: down(act(gate(x)) * up(x)), act = silu (SwiGLU) or the tanh form of gelu.
 
 gate and up are concatenated at load into one [2I, H] weight, the product lands in a
 packed [T, 2I] buffer and one kernel applies silu(g) * u (reference: MLP::forward,
@@ -25,32 +25,44 @@ class GatedMLP(FeedForward):
         super().__init__(spec, dtype)
         self.hidden = int(spec["hidden_size"])
         self.inter = int(spec["intermediate_size"])
-        if spec.get("activation", "silu") != "silu":
-            raise NotImplementedError(f"activation {spec.get('activation')!r} is not built (silu only)")
+        self.activation = str(spec.get("activation", "silu"))
+        if self.activation not in kernels.ACTIVATIONS:
+            raise NotImplementedError(f"activation {self.activation!r} is not built ({', '.join(kernels.ACTIVATIONS)})")
         self.gate_up: Optional[Linear] = None
         self.down: Optional[Linear] = None
+
+    NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
+
+    @classmethod
+    def _names(cls, spec: PartSpec, prefix: str):
+        """The three tensors' names: the spec's `names` (what follows the prefix) over the defaults."""
+        given = spec.get("names") or {}
+        return {k: f"{prefix}.{given.get(k, v)}" for k, v in cls.NAMES.items()}
 
     @classmethod
     def declare(cls, spec: PartSpec, prefix: str) -> List[TensorDecl]:
         h, i = int(spec["hidden_size"]), int(spec["intermediate_size"])
-        return [TensorDecl(f"{prefix}.gate_proj.weight", (i, h)),
-                TensorDecl(f"{prefix}.up_proj.weight", (i, h)),
-                TensorDecl(f"{prefix}.down_proj.weight", (h, i))]
+        n = cls._names(spec, prefix)
+        return [TensorDecl(n["gate"], (i, h)), TensorDecl(n["up"], (i, h)), TensorDecl(n["down"], (h, i))]
 
     def load(self, store: WeightStore, prefix: str, device) -> None:
         def lin(name):
             t = store.get(name, None, device)
             return t.to(self.dtype) if (self.dtype == torch.float32 or t.dtype != torch.float32) else t
-        g, u = lin(f"{prefix}.gate_proj.weight"), lin(f"{prefix}.up_proj.weight")
+        n = self._names(self.spec, prefix)
+        g, u = lin(n["gate"]), lin(n["up"])
         common = torch.float32 if torch.float32 in (g.dtype, u.dtype) else g.dtype
         self.gate_up = Linear(torch.cat([g.to(common), u.to(common)], dim=0))
-        self.down = Linear(lin(f"{prefix}.down_proj.weight"))
+        self.down = Linear(lin(n["down"]))
 
     takes_sink = True
     takes_folded = True
 
     def forward(self, x, ctx: StepContext, sink=None):
         """`x`: rows or a `Folded`; `sink`: see `Part.takes_sink`."""
+        if self.activation != "silu":        # the fused products apply silu; other activations take two steps
+            m = kernels.act_mul(self.gate_up(x, out_dtype=self.dtype), self.activation)
+            return self.down(m, out_dtype=self.dtype, allow_split=True, sink=sink)
         m = self.gate_up(x, out_dtype=self.dtype, gated=True)         # gate, up and silu*mul in one pass
         if m is None:
             m = kernels.silu_mul(self.gate_up(x, out_dtype=self.dtype))

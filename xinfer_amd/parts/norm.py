@@ -39,3 +39,6 @@ class RMSNorm(Norm):
 
     def forward(self, resid, add, out_dtype, rows=None, out=None):
         return kernels.add_rmsnorm(resid, add, self.weight, self.eps, out_dtype, rows=rows, out=out)
+
+    def forward_branch(self, resid, y, rows_dtype):
+        return kernels.rmsnorm_add(resid, y, self.weight, self.eps, rows_dtype)

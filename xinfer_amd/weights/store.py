@@ -57,7 +57,8 @@ class WeightError(RuntimeError):
 @dataclass(frozen=True)
 class TensorDecl:
     """A tensor a part needs.  `init` names how random weights fill it:
-    "linear" ~ N(0, linear_std), "norm" ~ 1 + N(0, norm_std), "zeros"."""
+    "linear" ~ N(0, linear_std), "norm" ~ 1 + N(0, norm_std), "mix" ~ 0.5 + N(0, norm_std) (a blend's
+    scalar), "zeros"."""
     name: str
     shape: Tuple[int, ...]
     init: str = "linear"
@@ -192,6 +193,8 @@ class RandomStore(WeightStore):
             return torch.zeros(d.shape, dtype=self.dtype, device=dev)
         if d.init == "norm":
             scale, shift = self.norm_std, 1.0
+        elif d.init == "mix":
+            scale, shift = self.norm_std, 0.5
         elif d.init == "linear":
             scale, shift = self.linear_std, 0.0
         else:
