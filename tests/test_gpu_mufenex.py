@@ -224,6 +224,40 @@ def test_attention_generic_kernel_with_planted_keys(case, dtype):
     _attention_case(case, dtype, fn)
 
 
+@pytest.mark.parametrize("small", [None, 0, 1])
+@pytest.mark.parametrize("case", ATTN_CASES + [(8, 1, 256, 128, 70, 25.0, 0.0625, 210), (2, 2, 32, 256, None, 25.0, 0.2, 190)])
+def test_attention_matrix_core_kernel_with_planted_keys(case, small):
+    """The bfloat16 kernel for scores with options: the same planted sequences, as a portion and token by
+    token, in both workgroup shapes; also beside the generic kernel on the same operands."""
+    from xinfer_amd import kernels
+    H, G, d, dv = case[:4]
+    assert kernels.attention_biased_supported(H, G, d, dv, 16)
+
+    def fn(q, k_pool, v_pool, table, positions, scale, window, grouped, softcap, slopes):
+        n, ctx = len(positions), positions[-1] + 1
+        cu_q = torch.tensor([0, n], dtype=torch.int32, device=DEV)
+        ctx_lens = torch.tensor([ctx], dtype=torch.int32, device=DEV)
+        rows, shape = kernels.prefill_tiles([n], [ctx], d, H, G, small=small,
+                                            block_of=lambda s_: kernels.attention_biased_block(d, dv, H // G, s_))
+        tiles = torch.tensor(rows, dtype=torch.int32, device=DEV).reshape(-1, 2)
+        out = kernels.attention_biased_bf16(q, k_pool, v_pool, table, tiles, cu_q, ctx_lens, scale, window,
+                                            softcap=softcap, slopes=slopes, small=shape)
+        pos = torch.tensor(positions, dtype=torch.int32, device=DEV)
+        ref = kernels.attention_generic(q, k_pool, v_pool, table, torch.zeros_like(pos), pos, scale, window,
+                                        v_grouped=True, softcap=softcap, slopes=slopes)
+        assert (out.float() - ref.float()).abs().max() <= 0.03 * ref.float().abs().max()
+        return out
+    _attention_case(case, "bfloat16", fn)
+
+
+def test_sizes_the_matrix_core_kernel_does_not_take():
+    from xinfer_amd import kernels
+    assert not kernels.attention_biased_supported(4, 4, 16, 12, 16)       # a value size that is no multiple of 8
+    assert not kernels.attention_biased_supported(4, 4, 264, 16, 16)
+    assert not kernels.attention_biased_supported(4, 3, 16, 16, 16)
+    assert not kernels.attention_biased_supported(4, 4, 16, 16, 12)
+
+
 def test_attention_without_the_options_is_the_plain_softmax():
     """No cap and no slopes: the kernel's options are off, not zero-valued."""
     from xinfer_amd import kernels

@@ -604,7 +604,7 @@ MIXED_DECODE_CONTEXT = 4096    # or the longest context this (measured on MI355X
                                # 40 query heads on 8 kv heads, 64 sequences at 1,500 keys: 450 -> 155 us a layer)
 
 
-def prefill_tiles(q_lens, ctx_lens, d: int, nq: int, nkv: int, small=None, first_seq: int = 0):
+def prefill_tiles(q_lens, ctx_lens, d: int, nq: int, nkv: int, small=None, first_seq: int = 0, block_of=None):
     """The query blocks of a batch of portions for the prefill kernel: (rows, shape).
     rows = [(sequence, first query of the block)] in launch order.  A block's work grows
     with the keys it sees, and the compute units take workgroups in launch order, so the
@@ -620,16 +620,19 @@ def prefill_tiles(q_lens, ctx_lens, d: int, nq: int, nkv: int, small=None, first
     workgroup per unit at a time: longest first."""
     g = nq // nkv
     heads = nkv * (g // (4 if g % 4 == 0 else 2 if g % 2 == 0 else 1))     # workgroups per query block
-    big = prefill_block(d, g, False)
+    two_groups = block_of is None          # (`block_of(small)`: another kernel's block sizes, shapes 0 and 1 only)
+    if block_of is None:
+        block_of = lambda shape: prefill_block(d, g, shape)
+    big = block_of(0)
     if small is None:
         blocks = sum(-(-n // big) for n in q_lens[first_seq:])
         small = 0 if blocks * heads >= 2 * COMPUTE_UNITS else 1
-        if small and PREFILL_RING and prefill_ring_supported(d):
-            half = prefill_block(d, g, 1)
+        if small and two_groups and PREFILL_RING and prefill_ring_supported(d):
+            half = block_of(1)
             if sum(-(-n // half) for n in q_lens[first_seq:]) * heads <= 2 * COMPUTE_UNITS:
                 small = 2
     small = int(small)
-    qb = prefill_block(d, g, small)
+    qb = block_of(small)
     rows = [(b, q0) for b, n in enumerate(q_lens) if b >= first_seq for q0 in range(0, n, qb)]
     rows.sort(key=lambda t: -(ctx_lens[t[0]] - q_lens[t[0]] + t[1]))
     per_round = max(1, COMPUTE_UNITS // heads)
@@ -638,6 +641,54 @@ def prefill_tiles(q_lens, ctx_lens, d: int, nq: int, nkv: int, small=None, first
         chunk = rows[i:i + per_round]
         out += chunk if (small != 1 or (i // per_round) % 2 == 0) else chunk[::-1]
     return out, small
+
+
+BIASED_MFMA = True        # False: scores with options go to the generic kernel in bfloat16 too
+
+
+def attention_biased_supported(nq: int, nkv: int, d: int, dv: int, page: int) -> bool:
+    return bool(lib().xi_attention_biased_supported(int(nq), int(nkv), int(d), int(dv), int(page)))
+
+
+def attention_biased_block(d: int, dv: int, group: int = 1, small: int = 0) -> int:
+    """Query positions per workgroup of `attention_biased_bf16` for the two head sizes, a number of
+    query heads per kv head and a workgroup shape (0: eight waves, 1: four)."""
+    return int(lib().xi_attention_biased_block(int(d), int(dv), int(group), int(small)))
+
+
+def attention_biased_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, scale, window=0, softcap=0.0,
+                          slopes=None, out=None, small=0):
+    """Matrix-core attention for any mix of portions with the score's options (`softcap`, `slopes`: see
+    `attention_generic`) and a value head size of its own: q [T, nq, d], K pool [pages, nkv, page, d], V pool
+    [pages, nkv, page / 8, dv, 8]; tiles int32 [n, 2] = (sequence, first query token of a block of
+    `attention_biased_block(d, dv, nq // nkv, small)` tokens within the sequence's portion).  Returns [T, nq * dv]."""
+    _dev(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, out, slopes)
+    T, nq, d = q.shape
+    nkv, page, dv = k_cache.shape[1], k_cache.shape[2], int(vt_cache.shape[3])
+    _want(q, torch.bfloat16, "attention_biased: q")
+    _check_cache(k_cache, vt_cache, nkv, d, torch.bfloat16, True, "attention_biased", dv=dv)
+    for t, name in ((block_tables, "block_tables"), (tiles, "tiles"), (cu_q, "cu_q"), (ctx_lens, "ctx_lens")):
+        _want(t, torch.int32, f"attention_biased: {name}")
+    B = ctx_lens.shape[0]
+    if block_tables.dim() != 2 or block_tables.shape[0] != B or cu_q.shape != (B + 1,) or tiles.dim() != 2 or tiles.shape[1] != 2:
+        raise KernelError("attention_biased: block_tables [B, pages], cu_q [B+1], ctx_lens [B], tiles [n, 2] expected")
+    if not attention_biased_supported(nq, nkv, d, dv, page):
+        raise KernelError(f"attention_biased: sizes nq={nq} nkv={nkv} d={d} dv={dv} page={page} are not taken")
+    if slopes is not None:
+        _want(slopes, torch.float32, "attention_biased: slopes")
+        if slopes.shape != (nq,):
+            raise KernelError(f"attention_biased: slopes {tuple(slopes.shape)} must be one a query head, [{nq}]")
+    if int(small) not in (0, 1) or not softcap >= 0:
+        raise KernelError("attention_biased: the shape is 0 or 1, the soft cap positive or 0")
+    if out is None:
+        out = torch.empty((T, nq * dv), dtype=q.dtype, device=q.device)
+    elif out.shape != (T, nq * dv) or out.dtype != q.dtype:
+        raise KernelError("attention_biased: out has the wrong shape or dtype")
+    _ok(lib().xi_attention_biased_bf16(
+        _p(q), _p(k_cache), _p(vt_cache), _p(block_tables), int(block_tables.shape[1]), _p(tiles), int(tiles.shape[0]),
+        _p(cu_q), _p(ctx_lens), _p(out), ctypes.c_float(scale), ctypes.c_float(softcap), _p(slopes), int(window), int(page),
+        nq, nkv, d, dv, int(small), _stream()))
+    return out
 
 
 def attention_decode_bf16(q, k_cache, vt_cache, block_tables, ctx_lens, max_ctx_len, scale, window=0, out=None,
@@ -738,6 +789,23 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx
     nkv, page = k_cache.shape[1], k_cache.shape[2]
     bt = ctx.block_tables[group]
     if softcap > 0 or slopes is not None or v_cache.shape[3] != d:
+        dv = int(v_cache.shape[3])
+        if q.dtype == torch.bfloat16 and v_grouped and BIASED_MFMA and attention_biased_supported(nq, nkv, d, dv, page):
+            key = ("attention_biased_tiles", d, dv, nq, nkv)
+            cached = ctx.scratch.get(key)
+            if cached is None:
+                if ctx.max_q_len == 1:       # a step of single tokens: a block a sequence, nothing of the step read here
+                    one = torch.arange(ctx.num_seqs, dtype=torch.int32, device=q.device)
+                    cached = (torch.stack([one, torch.zeros_like(one)], dim=1).contiguous(), 1)
+                else:
+                    q_lens = [ctx.cu_q_host[b + 1] - ctx.cu_q_host[b] for b in range(ctx.num_seqs)]
+                    rows, small = prefill_tiles(q_lens, ctx.ctx_lens_host, d, nq, nkv,
+                                                block_of=lambda shape: attention_biased_block(d, dv, nq // nkv, shape))
+                    cached = (torch.tensor(rows, dtype=torch.int32, device=q.device).reshape(-1, 2), small)
+                ctx.scratch[key] = cached
+            tiles, small = cached
+            return attention_biased_bf16(q, k_cache, v_cache, bt, tiles, ctx.cu_q, ctx.ctx_lens, scale, window,
+                                         softcap=softcap, slopes=slopes, small=small)
         return attention_generic(q, k_cache, v_cache, bt, ctx.tok_seq, ctx.positions, scale, window,
                                  v_grouped=v_grouped, softcap=softcap, slopes=slopes)
     if q.dtype == torch.bfloat16 and v_grouped and mfma_attention_supported(nq, nkv, d, page):
