@@ -313,6 +313,34 @@ def test_experts(E, top, H, F, T, dtype):
     assert (got.cpu().double() - want).abs().max() < tol * want.abs().max()
 
 
+@pytest.mark.parametrize("E,top,H,F,T", [(5, 2, 96, 48, 19), (3, 1, 104, 24, 5), (8, 2, 512, 128, 70), (4, 4, 64, 200, 1),
+                                         (16, 2, 256, 64, 700), (2, 1, 64, 64, 300), (64, 6, 128, 32, 33)])
+def test_experts_grouped_on_the_matrix_cores(E, top, H, F, T):
+    """The grouped form against the plain implementation and against a pair at a time: tiles that are full, ragged
+    and empty (experts nobody chose), both tile heights."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(F + T)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    W = {"r.router": torch.randn(E, H, generator=g) * 0.3, "r.router.b": torch.randn(E, generator=g)}
+    if E == 16:
+        W["r.router.b"][3] = -100.0          # an expert without rows
+    for e in range(E):
+        W[f"r.e{e}.gate"] = (torch.randn(F, H, generator=g) * 0.1).to(torch.bfloat16)
+        W[f"r.e{e}.up"] = (torch.randn(F, H, generator=g) * 0.1).to(torch.bfloat16)
+        W[f"r.e{e}.down"] = (torch.randn(H, F, generator=g) * 0.1).to(torch.bfloat16)
+    gi, gw = kernels.moe_route(x.to(DEV), W["r.router"].to(DEV), W["r.router.b"].to(DEV), top)
+    gu = torch.stack([torch.cat([W[f"r.e{e}.gate"], W[f"r.e{e}.up"]]) for e in range(E)]).to(DEV)
+    dn = torch.stack([W[f"r.e{e}.down"] for e in range(E)]).to(DEV)
+    one = kernels.moe_experts(x.to(DEV), gu, dn, gi, gw, "silu", grouped=False)
+    got = kernels.moe_experts(x.to(DEV), gu, dn, gi, gw, "silu", grouped=True)
+    assert (got - one).abs().max() <= 0.02 * one.abs().max()
+    if T <= 100:
+        want = plain.experts_ff(x.double(), {k: t.double() for k, t in W.items()}, "r.", {"router": {"experts": E, "top": top}})
+        assert (got.cpu().double() - want).abs().max() < 2e-2 * want.abs().max()
+    assert not kernels.moe_grouped_takes(T, top, E, H + 4, F, torch.bfloat16, force=True)
+    assert not kernels.moe_grouped_takes(T, top, E, H, F, torch.float32, force=True)
+
+
 # ---- whole models ---------------------------------------------------------------------------------
 LENGTHS = {"P": [1, 2, 12, 13, 33, 77, 130], "Q": [3, 9, 10, 18, 64, 101], "R": [5, 101, 330, 64, 301]}
 

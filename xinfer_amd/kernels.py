@@ -312,12 +312,25 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor
     return idx, wt
 
 
+MOE_GROUPED = True        # False: every step takes the experts one (token, expert) pair at a time
+
+
+def moe_grouped_takes(T: int, top: int, E: int, H: int, F: int, dtype: torch.dtype, force: bool = False) -> bool:
+    """Whether a step's experts go through the grouped matrix-core products: bfloat16, sizes in eights,
+    and more pairs than experts (with fewer, most pairs have an expert of their own and a pair at a time
+    reads no more weights, in two launches instead of four); `force`: only whether the sizes are taken."""
+    if dtype != torch.bfloat16 or H % 8 or F % 8 or E > 1024 or T < 1:
+        return False
+    return force or (MOE_GROUPED and T * top > E)
+
+
 def moe_experts(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx: torch.Tensor, wt: torch.Tensor,
-                act: str = "silu") -> torch.Tensor:
+                act: str = "silu", grouped: Optional[bool] = None) -> torch.Tensor:
     """sum over a token's chosen experts e (in the order of `idx`) of wt * down[e] @ (act(gate[e] @ x) * (up[e] @ x)):
     gate_up [E, 2F, H] (gate rows first), down [E, H, F], idx int32 / wt float32 [T, top].  Float32 [T, H].
     One (token, expert) pair at a time, every sum in an order fixed by the sizes: the form of the
-    float32 path and of steps with few tokens."""
+    float32 path and of steps with few tokens.  `grouped` (None: chosen by `moe_grouped_takes`): the pairs
+    sorted by expert on the device and each expert's rows multiplied in tiles on the matrix cores."""
     _dev(x, gate_up, down, idx, wt)
     if act not in ACTIVATIONS:
         raise KernelError(f"moe_experts: unknown activation {act!r}")
@@ -334,8 +347,29 @@ def moe_experts(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx:
     if idx.dim() != 2 or idx.shape[0] != T or wt.shape != idx.shape:
         raise KernelError("moe_experts: idx and weights must be [T, top]")
     top = int(idx.shape[1])
-    mid = torch.empty((T * top, F), dtype=x.dtype, device=x.device)
     out = torch.empty((T, H), dtype=torch.float32, device=x.device)
+    if grouped is None:
+        grouped = moe_grouped_takes(T, top, E, H, F, x.dtype)
+    if grouped:
+        if not moe_grouped_takes(T, top, E, H, F, x.dtype, force=True):
+            raise KernelError(f"moe_experts: the grouped form takes bfloat16 and sizes in eights, not {x.dtype} H={H} F={F}")
+        P = T * top
+        bm = 64 if P >= 48 * E else 32               # rows of a tile: 64 where most experts fill them
+        most = int(lib().xi_moe_tiles_most(P, E, bm))
+        ints = torch.empty((2 * P + 3 * most + 1,), dtype=torch.int32, device=x.device)
+        order, slot_of = ints[:P], ints[P:2 * P]
+        t_e, t_r0, t_n, n_tiles = (ints[2 * P:2 * P + most], ints[2 * P + most:2 * P + 2 * most],
+                                   ints[2 * P + 2 * most:2 * P + 3 * most], ints[2 * P + 3 * most:])
+        _ok(lib().xi_moe_sort(_p(idx), P, E, bm, _p(order), _p(slot_of), _p(t_e), _p(t_r0), _p(t_n), _p(n_tiles), _stream()))
+        mid = torch.empty((P, F), dtype=torch.bfloat16, device=x.device)
+        _ok(lib().xi_moe_group(_p(x), _p(order), top, _p(gate_up), _p(t_e), _p(t_r0), _p(t_n), _p(n_tiles), most, _p(mid),
+                               F, H, bm, 1, ACTIVATIONS[act], _stream()))
+        y = torch.empty((P, H), dtype=torch.float32, device=x.device)
+        _ok(lib().xi_moe_group(_p(mid), _p(order), top, _p(down), _p(t_e), _p(t_r0), _p(t_n), _p(n_tiles), most, _p(y),
+                               H, F, bm, 0, 0, _stream()))
+        _ok(lib().xi_moe_combine(_p(y), _p(slot_of), _p(wt), _p(out), T, H, top, _stream()))
+        return out
+    mid = torch.empty((T * top, F), dtype=x.dtype, device=x.device)
     code = _code(x, "moe_experts")
     _ok(lib().xi_moe_gate_up(_p(x), _p(gate_up), _p(idx), _p(mid), code, ACTIVATIONS[act], T, H, F, E, top, _stream()))
     _ok(lib().xi_moe_down(_p(mid), _p(down), _p(idx), _p(wt), _p(out), code, T, H, F, E, top, _stream()))
