@@ -31,6 +31,11 @@ batching, greedy sampling) and print their own JSON line: total generated tokens
 concurrent requests, 1,024 new tokens each); its line carries the ratio to that figure, which
 was measured on other hardware.  `--workload many8b` is 192 concurrent requests (prompts of 64
 to 512 tokens, 256 new tokens each) at Qwen3-8B sizes: decode steps of 129 to 256 rows.
+
+`--design mufenex[:SIZE]` times the Mufenex family (windowed attention with a soft cap and a distance
+bias, sublayer outputs normed, dense gelu or routed silu feed-forwards) beside Qwen3 at equal sizes
+(the same width, heads, head size, feed-forward width, window, vocabulary and number of layers): the
+prefill of one prompt and a decode step at batch 8, one JSON line with both.
 """
 from __future__ import annotations
 
@@ -67,6 +72,15 @@ WORKLOADS = {
     "long32b": dict(model=QWEN3_32B, name="Qwen3-32B layer sizes", requests=16, prompt=(8192, 8192), new_tokens=512,
                     chunk=2048, max_model_len=8704),
 }
+# sizes of the `--design` comparison: width, query heads, kv heads, head size, value head size, feed-forward width,
+# window, experts (0: dense; else `experts` of `top`, each of ff / top so that a token's active width is ff)
+DESIGN_SIZES = {
+    "1k": dict(width=1024, heads=16, kv_heads=8, dim=128, vdim=128, ff=3072, window=1024, experts=0, top=0),
+    "4k": dict(width=4096, heads=32, kv_heads=8, dim=128, vdim=128, ff=12288, window=2048, experts=0, top=0),
+    "4k-moe": dict(width=4096, heads=32, kv_heads=8, dim=128, vdim=128, ff=12288, window=2048, experts=8, top=2),
+    "2k-v": dict(width=2048, heads=16, kv_heads=4, dim=64, vdim=128, ff=8192, window=512, experts=16, top=2),
+}
+DESIGN_VOCAB = 32000
 MODELS = {"0.6b": QWEN3_0_6B, "8b": QWEN3_8B, "14b": QWEN3_14B, "32b": QWEN3_32B}
 CONTEXT = 4096
 PREFILL_TOKENS = 2048
@@ -201,6 +215,108 @@ def product(spec: str, dev="cuda:0") -> int:
     return 0
 
 
+def design_compare(spec: str, layers, steps: int, warmup: int, batch: int, context: int, prefill_tokens: int,
+                   family: str = "both", only: str = "all") -> int:
+    """Mufenex beside Qwen3 at equal sizes: ms of the prefill of one prompt and of a decode step."""
+    import torch
+    from xinfer_amd.engine import ModelRunner, StepEntry, build_model
+    from xinfer_amd.models import config_from_dict
+    from xinfer_amd.sampling import Sampler
+    from xinfer_amd.weights.random_init import random_store_for
+    name, _, size = spec.partition(":")
+    if name != "mufenex" or (size and size not in DESIGN_SIZES):
+        print(f"bench.py: --design mufenex[:{'|'.join(DESIGN_SIZES)}]")
+        return 2
+    dev, page = "cuda:0", 64
+    layers = layers or 4
+    sampler = Sampler(dev)
+    gen = torch.Generator().manual_seed(3)
+    out = {"metric": "Mufenex beside Qwen3 at equal sizes, bf16", "unit": "ms", "layers": layers, "batch": batch,
+           "context": context, "prefill_tokens": prefill_tokens, "data": "synthetic: seeded random weights and token ids",
+           "sizes": {}}
+
+    def configs(z):
+        mixer = dict(dim=z["dim"], heads=z["heads"], kv_heads=z["kv_heads"], vdim=z["vdim"], scale=z["dim"] ** -0.5,
+                     softcap=50.0, mask={"size": z["window"]}, v_mix=True)
+        mlp = ({"kind": "dense", "ff": z["ff"]} if not z["experts"] else
+               {"kind": "moe", "expert": {"ff": z["ff"] // z["top"]}, "router": {"experts": z["experts"], "top": z["top"]}})
+        mufenex = {"architecture": "Mufenex", "vocab": DESIGN_VOCAB, "width": z["width"], "embedding": {"scale": 1.0},
+                   "norm": {"eps": 1e-6}, "logit_softcap": 30.0, "max_positions": 2 * context,
+                   "layers": [{"type": "attention", "mixer": mixer, "mlp": mlp} for _ in range(layers)]}
+        qwen3 = dict(QWEN3_8B, hidden_size=z["width"], intermediate_size=z["ff"], num_hidden_layers=layers,
+                     num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"], head_dim=z["dim"],
+                     vocab_size=DESIGN_VOCAB, sliding_window=z["window"], max_position_embeddings=2 * context)
+        return {"mufenex": mufenex, "qwen3": qwen3}
+
+    def time_model(raw):
+        _, cfg = config_from_dict(raw)
+        model = build_model(cfg, random_store_for(cfg, seed=0, linear_std=0.02, norm_std=0.1), "bf16", dev)
+        pages = batch * (-(-context // page) + 2) + -(-prefill_tokens // page) + 8
+        runner = ModelRunner(model, page_size=page, num_pages=pages, max_requests=batch + 1)
+        g = torch.Generator(device=dev).manual_seed(1)
+        for lc in runner.layer_caches.values():
+            for t in lc.pools.values():
+                t.copy_(torch.randn(t.shape, generator=g, device=dev, dtype=torch.float32).to(t.dtype))
+        vocab = model.spec.vocab_size
+        ids = torch.randint(0, vocab, (prefill_tokens,), generator=gen).tolist()
+        best = None
+        for _ in range(4 if only != "decode" else 0):      # the first run warms up
+            runner.add_request(7)
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            sampler.argmax(runner.step([StepEntry(7, ids, [prefill_tokens - 1])])).tolist()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t
+            runner.release(7)
+            best = dt if best is None else min(best, dt)
+        if only == "prefill":
+            return {"prefill_ms": round(best * 1e3, 3), "prefill_tok_s": round(prefill_tokens / best, 1)}
+        prep = runner.graph_after
+        start = context - steps - warmup - prep
+        rids = list(range(100, 100 + batch))
+        for rid in rids:
+            runner.add_request(rid)
+            runner.cache.reserve(rid, start)
+            runner.cache.commit(rid, start)
+        places = list(range(batch))
+        prev = None
+
+        def one(prev):
+            if prev is None:
+                toks = torch.randint(0, vocab, (batch,), generator=gen).tolist()
+                logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(rids, toks)])
+            else:
+                logits = runner.step([StepEntry(r, [0], [0]) for r in rids], device_tokens=(prev, places, places))
+            return sampler.argmax(logits)
+        for _ in range(prep + warmup):
+            prev = one(prev)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            prev = one(prev)
+        torch.cuda.synchronize()
+        dec = (time.perf_counter() - t) / steps
+        assert 0 <= int(prev.min()) and int(prev.max()) < vocab
+        replays = runner.graph_replays
+        del runner, model
+        torch.cuda.empty_cache()
+        res = {"decode_ms": round(dec * 1e3, 4), "decode_tok_s": round(batch / dec, 1), "graph_replays": replays}
+        if best is not None:
+            res.update({"prefill_ms": round(best * 1e3, 3), "prefill_tok_s": round(prefill_tokens / best, 1)})
+        return res
+
+    for key in ([size] if size else list(DESIGN_SIZES)):
+        z = DESIGN_SIZES[key]
+        res = {k: time_model(raw) for k, raw in configs(z).items() if family in ("both", k)}
+        for what in ("prefill", "decode"):
+            if family == "both" and f"{what}_ms" in res["mufenex"]:
+                res[f"ratio_{what}"] = round(res["mufenex"][f"{what}_ms"] / res["qwen3"][f"{what}_ms"], 3)
+        out["sizes"][key] = dict(z, **res)
+        print(f"[bench] {key}: {res}", file=sys.stderr, flush=True)
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def measured_peaks(dev="cuda:0"):
     """(GB/s of a read-only stream over 4 GiB, TFLOP/s of one square bfloat16 product of 8192 in the
     vendor library): what this card reaches, beside the published peaks.  Best of five runs each."""
@@ -260,6 +376,11 @@ def main() -> int:
                     help="serving workloads: read every step's tokens on the host before the next step is planned")
     ap.add_argument("--product", default=None, metavar="M,N,K[,slices[,shape]]",
                     help="time one bfloat16 product alone in the many-row tiled kernel and in the vendor library")
+    ap.add_argument("--design", default=None, metavar="mufenex[:SIZE]",
+                    help="time another model family beside Qwen3 at equal sizes (a line of its own; --layers, --steps, "
+                         "--warmup, --batch, --context, --prefill-tokens and --only apply)")
+    ap.add_argument("--family", choices=["both", "mufenex", "qwen3"], default="both",
+                    help="--design: time one of the two families only (for profiling)")
     ap.add_argument("--peaks", action="store_true",
                     help="also measure what this card reaches on a read-only stream of 4 GiB and on one square "
                          "bfloat16 product of 8192, and report the fractions of those beside the fractions of the "
@@ -270,6 +391,9 @@ def main() -> int:
         return 2
     if args.product:
         return product(args.product)
+    if args.design:
+        return design_compare(args.design, args.layers, args.steps, args.warmup, args.batch, args.context, args.prefill_tokens,
+                              args.family, args.only)
     if args.workload != "decode":
         return serve(args.workload, args.layers, not args.no_run_ahead)
     full_layers = MODELS[args.model]["num_hidden_layers"]

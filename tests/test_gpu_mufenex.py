@@ -240,14 +240,26 @@ def test_attention_matrix_core_kernel_with_planted_keys(case, small):
         rows, shape = kernels.prefill_tiles([n], [ctx], d, H, G, small=small,
                                             block_of=lambda s_: kernels.attention_biased_block(d, dv, H // G, s_))
         tiles = torch.tensor(rows, dtype=torch.int32, device=DEV).reshape(-1, 2)
+        split, span = 0, 0
+        if n == 1 and small != 0:            # single tokens: also in slices of 64 or 128 keys put together afterwards
+            span = min(ctx, window + 63) if window else ctx
+            split = 64 if small is None else 128
         out = kernels.attention_biased_bf16(q, k_pool, v_pool, table, tiles, cu_q, ctx_lens, scale, window,
-                                            softcap=softcap, slopes=slopes, small=shape)
+                                            softcap=softcap, slopes=slopes, small=shape, split_keys=split, span=span)
         pos = torch.tensor(positions, dtype=torch.int32, device=DEV)
         ref = kernels.attention_generic(q, k_pool, v_pool, table, torch.zeros_like(pos), pos, scale, window,
                                         v_grouped=True, softcap=softcap, slopes=slopes)
         assert (out.float() - ref.float()).abs().max() <= 0.03 * ref.float().abs().max()
         return out
     _attention_case(case, "bfloat16", fn)
+
+
+def test_slices_of_a_decode_step():
+    from xinfer_amd import kernels
+    assert kernels.biased_split_keys(1024, 4096) == 0                 # enough workgroups already
+    assert kernels.biased_split_keys(64, 2048 + 63) == 320            # 8 slices asked for, 64-key steps
+    assert kernels.biased_split_keys(8, 100) == 0                     # too few keys to cut
+    assert kernels.biased_split_keys(1, 100000) % 64 == 0
 
 
 def test_sizes_the_matrix_core_kernel_does_not_take():

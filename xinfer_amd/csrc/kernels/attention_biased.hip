@@ -43,7 +43,8 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ vt_cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tiles,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, bf16* __restrict__ out, float scale,
-    float softcap, const float* __restrict__ slopes, int window, int page_shift, int nq, int nkv, int d, int dv) {
+    float softcap, const float* __restrict__ slopes, int window, int page_shift, int nq, int nkv, int d, int dv,
+    float* __restrict__ part_o, float* __restrict__ part_ml, int split_keys, int max_splits) {
   const int page = 1 << page_shift;
   constexpr int NT = 64 * NWV;                    // threads
   constexpr int QB = 16 * (NWV * NQT / GH);       // query positions per workgroup
@@ -79,6 +80,21 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
   const int wg_first = pos0 + q0_blk, wg_last = wg_first + wg_nq - 1;
   const int wg_lo = (window > 0 && wg_first - window + 1 > 0) ? wg_first - window + 1 : 0;
   const int k_begin = wg_lo & ~(kKeysB - 1);
+  // split_keys > 0 (steps of single tokens): this workgroup walks one slice of the keys, slice
+  // blockIdx.z of `split_keys` keys, and leaves its sums unnormalized for the combine kernel
+  const int kt_begin = k_begin + (split_keys > 0 ? (int)blockIdx.z * split_keys : 0);
+  const int kt_end = split_keys > 0 ? min(wg_last, kt_begin + split_keys - 1) : wg_last;
+  if (split_keys > 0 && kt_begin > wg_last) {          // a slice past the sequence's keys: it says so and ends
+    for (int ct = 0; ct < NQT; ++ct) {
+      const int tile = (threadIdx.x >> 6) * NQT + ct;
+      if (tile < GH && (threadIdx.x & 63) == 0) {
+        float* ml = part_ml + (((size_t)q_begin * nq + h0 + tile) * max_splits + blockIdx.z) * 2;
+        ml[0] = -INFINITY;
+        ml[1] = 0.f;
+      }
+    }
+    return;
+  }
 
   // this wave's queries: the position blocks its tiles lie in
   const int pb_lo = (wave * NQT) / GH, pb_hi = (wave * NQT + NQT - 1) / GH;
@@ -177,15 +193,15 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
 
   const float cap2 = softcap > 0.f ? 2.f * kLog2eB / softcap : 0.f;
   __syncthreads();   // the block table is in LDS
-  fetch(k_begin);
+  fetch(kt_begin);
   stash(0);
   // every load so far (the queries among them) has landed before the loop starts, so that
   // inside it only the tile in flight is ever waited for: vmcnt(0), other counters untouched
   __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();
   int buf = 0;
-  for (int kt = k_begin; kt <= wg_last; kt += kKeysB) {
-    const bool more = kt + kKeysB <= wg_last;
+  for (int kt = kt_begin; kt <= kt_end; kt += kKeysB) {
+    const bool more = kt + kKeysB <= kt_end;
     if (more) fetch(kt + kKeysB);
 #pragma unroll
     for (int sub = 0; sub < kKeysB / 32; ++sub) {
@@ -319,6 +335,20 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
     const int pb = tile / GH, hh = tile - pb * GH;
     const int qi = q0_blk + 16 * pb + r;
     if (qi >= q_len) continue;
+    if (split_keys > 0) {
+      const size_t at = ((size_t)(q_begin + qi) * nq + h0 + hh) * max_splits + blockIdx.z;
+      if (j == 0) {
+        part_ml[at * 2] = m_run[ct];
+        part_ml[at * 2 + 1] = lt;
+      }
+      float* po = part_o + at * dv;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        if (16 * dt + 4 * j >= dv) break;
+        *reinterpret_cast<f32x4*>(po + 16 * dt + 4 * j) = acc[dt][ct];
+      }
+      continue;
+    }
     const float inv = 1.f / lt;
     bf16* o = out + ((size_t)(q_begin + qi) * nq + h0 + hh) * dv;
 #pragma unroll
@@ -331,6 +361,31 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
       op[2] = __float2bfloat16(a[2] * inv);
       op[3] = __float2bfloat16(a[3] * inv);
     }
+  }
+}
+
+// Sums of the slices of a token's keys put together: out = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M), in slice
+// order (m_s: the slice's reference point in the exponent's unit; a slice without keys has m_s = -inf).
+__global__ __launch_bounds__(64) void attn_biased_combine_kernel(const float* __restrict__ part_o,
+                                                                 const float* __restrict__ part_ml, bf16* __restrict__ out,
+                                                                 int max_splits, int nq, int dv) {
+  const int head = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
+  const size_t base = ((size_t)t * nq + head) * max_splits;
+  float mm = -INFINITY;
+  for (int s2 = 0; s2 < max_splits; ++s2) mm = fmaxf(mm, part_ml[(base + s2) * 2]);
+  float ll = 0.f;
+  for (int s2 = 0; s2 < max_splits; ++s2) {
+    const float ms = part_ml[(base + s2) * 2];
+    if (ms > -INFINITY) ll += part_ml[(base + s2) * 2 + 1] * __builtin_amdgcn_exp2f(ms - mm);
+  }
+  const float inv = 1.f / ll;
+  for (int i = lane; i < dv; i += 64) {
+    float o = 0.f;
+    for (int s2 = 0; s2 < max_splits; ++s2) {
+      const float ms = part_ml[(base + s2) * 2];
+      if (ms > -INFINITY) o += part_o[(base + s2) * dv + i] * __builtin_amdgcn_exp2f(ms - mm);
+    }
+    out[((size_t)t * nq + head) * dv + i] = __float2bfloat16(o * inv);
   }
 }
 
@@ -364,15 +419,22 @@ int xi_attention_biased_block(int d, int dv, int g, int small) {
 int xi_attention_biased_bf16(const void* q, const void* k_cache, const void* vt_cache, const int* block_tables,
                              int max_pages, const int* tiles, int n_tiles, const int* cu_q, const int* ctx_lens,
                              void* out, float scale, float softcap, const float* slopes, int window, int page, int nq,
-                             int nkv, int d, int dv, int small, hipStream_t stream) {
+                             int nkv, int d, int dv, int small, float* part_o, float* part_ml, int split_keys,
+                             int max_splits, int n_tok, hipStream_t stream) {
   XI_CHECK(xi_attention_biased_supported(nq, nkv, d, dv, page), "attention_biased: unsupported sizes nq=%d nkv=%d d=%d dv=%d page=%d",
            nq, nkv, d, dv, page);
   XI_CHECK(n_tiles >= 0 && n_tiles <= 65535, "attention_biased: %d query blocks are too many for one launch", n_tiles);
   XI_CHECK(softcap >= 0.f, "attention_biased: the soft cap must be positive (0: none)");
+  // slices of the keys: for steps in which every sequence brings one token (a tile a token), partial sums
+  // part_o float32 [n_tok, nq, max_splits, dv] and part_ml [n_tok, nq, max_splits, 2] from the caller
+  XI_CHECK(split_keys == 0 || (split_keys > 0 && split_keys % kKeysB == 0 && max_splits > 0 && max_splits <= 65535 &&
+                               part_o != nullptr && part_ml != nullptr && n_tiles == n_tok && dv % 4 == 0),
+           "attention_biased: slices of %d keys (%d of them) need steps of single tokens and room for the partial sums",
+           split_keys, max_splits);
   if (n_tiles == 0) return 0;
   const int g = nq / nkv;
   const int gh = heads_together_b(g);
-  dim3 grid(nkv * (g / gh), n_tiles);
+  dim3 grid(nkv * (g / gh), n_tiles, split_keys > 0 ? max_splits : 1);
   int page_shift = -1;
   for (int b = 0; b < 31; ++b)
     if ((1 << b) == page) page_shift = b;
@@ -391,7 +453,8 @@ int xi_attention_biased_bf16(const void* q, const void* k_cache, const void* vt_
     }                                                                                                   \
     kern<<<grid, 64 * NWV, lds, stream>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)vt_cache,  \
                                           block_tables, max_pages, tiles, cu_q, ctx_lens, (bf16*)out,   \
-                                          scale, softcap, slopes, window, page_shift, nq, nkv, d, dv);  \
+                                          scale, softcap, slopes, window, page_shift, nq, nkv, d, dv,   \
+                                          part_o, part_ml, split_keys, max_splits);                     \
   } while (0)
 #define XI_PB_GH(KC, DT, NQT, NWV)             \
   do {                                         \
@@ -429,6 +492,10 @@ int xi_attention_biased_bf16(const void* q, const void* k_cache, const void* vt_
 #undef XI_PB_GH
 #undef XI_PB
   XI_LAUNCH_CHECK("attention_biased");
+  if (split_keys > 0) {
+    attn_biased_combine_kernel<<<dim3(nq, n_tok), 64, 0, stream>>>(part_o, part_ml, (bf16*)out, max_splits, nq, dv);
+    XI_LAUNCH_CHECK("attention_biased_combine");
+  }
   return 0;
 }
 

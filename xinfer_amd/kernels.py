@@ -690,12 +690,29 @@ def attention_biased_block(d: int, dv: int, group: int = 1, small: int = 0) -> i
     return int(lib().xi_attention_biased_block(int(d), int(dv), int(group), int(small)))
 
 
+BIASED_SPLIT_WORKGROUPS = 512     # workgroups a launch of single tokens aims at (two a compute unit)
+BIASED_SPLIT_KEYS_LEAST = 128     # keys of a slice at least
+
+
+def biased_split_keys(workgroups: int, span: int) -> int:
+    """Keys a slice (a multiple of 64; 0: no slices) for a step of single tokens that would make `workgroups`
+    workgroups, each walking up to `span` keys: slices until the launch has about BIASED_SPLIT_WORKGROUPS."""
+    want = BIASED_SPLIT_WORKGROUPS // max(1, int(workgroups))
+    most = int(span) // BIASED_SPLIT_KEYS_LEAST
+    splits = min(want, most)
+    if splits < 2:
+        return 0
+    return -(-int(span) // splits // 64) * 64
+
+
 def attention_biased_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, scale, window=0, softcap=0.0,
-                          slopes=None, out=None, small=0):
+                          slopes=None, out=None, small=0, split_keys=0, span=0):
     """Matrix-core attention for any mix of portions with the score's options (`softcap`, `slopes`: see
     `attention_generic`) and a value head size of its own: q [T, nq, d], K pool [pages, nkv, page, d], V pool
     [pages, nkv, page / 8, dv, 8]; tiles int32 [n, 2] = (sequence, first query token of a block of
-    `attention_biased_block(d, dv, nq // nkv, small)` tokens within the sequence's portion).  Returns [T, nq * dv]."""
+    `attention_biased_block(d, dv, nq // nkv, small)` tokens within the sequence's portion).  Returns [T, nq * dv].
+    `split_keys` > 0 (steps in which every sequence brings one token, a tile a token): each workgroup walks one slice
+    of that many keys of the up to `span` a token sees, and a second kernel puts the slices together."""
     _dev(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, out, slopes)
     T, nq, d = q.shape
     nkv, page, dv = k_cache.shape[1], k_cache.shape[2], int(vt_cache.shape[3])
@@ -718,10 +735,18 @@ def attention_biased_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_l
         out = torch.empty((T, nq * dv), dtype=q.dtype, device=q.device)
     elif out.shape != (T, nq * dv) or out.dtype != q.dtype:
         raise KernelError("attention_biased: out has the wrong shape or dtype")
+    part_o = part_ml = None
+    max_splits = 0
+    if split_keys:
+        if split_keys % 64 or split_keys < 0 or span <= 0 or tiles.shape[0] != T or B != T:
+            raise KernelError("attention_biased: slices are multiples of 64 keys, for steps of single tokens with a tile each")
+        max_splits = (int(span) + 63) // int(split_keys) + 1
+        part_o = torch.empty((T, nq, max_splits, dv), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((T, nq, max_splits, 2), dtype=torch.float32, device=q.device)
     _ok(lib().xi_attention_biased_bf16(
         _p(q), _p(k_cache), _p(vt_cache), _p(block_tables), int(block_tables.shape[1]), _p(tiles), int(tiles.shape[0]),
         _p(cu_q), _p(ctx_lens), _p(out), ctypes.c_float(scale), ctypes.c_float(softcap), _p(slopes), int(window), int(page),
-        nq, nkv, d, dv, int(small), _stream()))
+        nq, nkv, d, dv, int(small), _p(part_o), _p(part_ml), int(split_keys), int(max_splits), int(T), _stream()))
     return out
 
 
@@ -838,8 +863,13 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx
                     cached = (torch.tensor(rows, dtype=torch.int32, device=q.device).reshape(-1, 2), small)
                 ctx.scratch[key] = cached
             tiles, small = cached
+            split, span = 0, 0
+            if ctx.max_q_len == 1:           # single tokens: slices of the keys where the sequences alone leave the chip idle
+                g = nq // nkv
+                span = min(int(ctx.max_ctx_len), int(window) + 63) if window > 0 else int(ctx.max_ctx_len)
+                split = biased_split_keys(ctx.num_seqs * nkv * (g // (4 if g % 4 == 0 else 2 if g % 2 == 0 else 1)), span)
             return attention_biased_bf16(q, k_cache, v_cache, bt, tiles, ctx.cu_q, ctx.ctx_lens, scale, window,
-                                         softcap=softcap, slopes=slopes, small=small)
+                                         softcap=softcap, slopes=slopes, small=small, split_keys=split, span=span)
         return attention_generic(q, k_cache, v_cache, bt, ctx.tok_seq, ctx.positions, scale, window,
                                  v_grouped=v_grouped, softcap=softcap, slopes=slopes)
     if q.dtype == torch.bfloat16 and v_grouped and mfma_attention_supported(nq, nkv, d, page):
