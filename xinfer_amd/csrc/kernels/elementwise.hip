@@ -529,6 +529,52 @@ __global__ __launch_bounds__(NT) void rmsnorm_add_kernel(float* __restrict__ res
   }
 }
 
+// The same for widths that are a multiple of 4 up to 4 * NT * MAXV: a thread keeps its part of the row in
+// registers, every operand is read once in 16-byte (bfloat16: 8-byte) pieces and all loads are in flight together.
+template <typename TY, typename TR, int NT, int MAXV>
+__global__ __launch_bounds__(NT) void rmsnorm_add_vec_kernel(float* __restrict__ resid, const TY* __restrict__ y, int parts,
+                                                             size_t part_stride, const float* __restrict__ w, float eps,
+                                                             TR* __restrict__ rows, int H) {
+  __shared__ float scratch[NT / kWave];
+  const int row = blockIdx.x;
+  float* x = resid + (size_t)row * H;
+  const TY* yr = y + (size_t)row * H;
+  float4 s[MAXV], xv[MAXV], wv[MAXV];
+  float ss = 0.f;
+#pragma unroll
+  for (int v = 0; v < MAXV; ++v) {
+    const int i = 4 * (threadIdx.x + NT * v);
+    if (i < H) {
+      s[v] = load4(yr + i);
+      xv[v] = load4(x + i);
+      wv[v] = w ? load4(w + i) : float4{1.f, 1.f, 1.f, 1.f};
+      for (int p = 1; p < parts; ++p) {
+        const float4 t = load4(yr + p * part_stride + i);
+        s[v].x += t.x;
+        s[v].y += t.y;
+        s[v].z += t.z;
+        s[v].w += t.w;
+      }
+      ss += s[v].x * s[v].x + s[v].y * s[v].y + s[v].z * s[v].z + s[v].w * s[v].w;
+    }
+  }
+  float inv = 1.f;
+  if (w) inv = rsqrtf(block_sum<NT / kWave>(ss, scratch) / (float)H + eps);
+#pragma unroll
+  for (int v = 0; v < MAXV; ++v) {
+    const int i = 4 * (threadIdx.x + NT * v);
+    if (i < H) {
+      float4 o;
+      o.x = xv[v].x + s[v].x * inv * wv[v].x;
+      o.y = xv[v].y + s[v].y * inv * wv[v].y;
+      o.z = xv[v].z + s[v].z * inv * wv[v].z;
+      o.w = xv[v].w + s[v].w * inv * wv[v].w;
+      store4(x + i, o);
+      if (rows) store4(rows + (size_t)row * H + i, o);
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------
 // act(gate) * up for a packed [T, 2I] buffer, the activation chosen by code:
 // 0 silu(z) = z * sigmoid(z); 1 the tanh form of gelu, 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
@@ -545,6 +591,87 @@ __global__ void act_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, in
     const size_t t = idx / I, i = idx - t * I;
     const float g = to_float(gu[t * 2 * I + i]), u = to_float(gu[t * 2 * I + I + i]);
     out[idx] = from_float<T>(act_of<ACT>(g) * u);
+  }
+}
+
+template <int ACT>
+__global__ void act_mul_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int I, size_t total8) {
+  const int I8 = I / 8;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total8; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / I8, i = (idx - t * I8) * 8;
+    const bf16x8_t g = *reinterpret_cast<const bf16x8_t*>(gu + t * 2 * I + i);
+    const bf16x8_t u = *reinterpret_cast<const bf16x8_t*>(gu + t * 2 * I + I + i);
+    bf16x8_t o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o.v[e] = from_float<bf16>(act_of<ACT>(to_float(g.v[e])) * to_float(u.v[e]));
+    *reinterpret_cast<bf16x8_t*>(out + t * I + i) = o;
+  }
+}
+
+// The projection rows' kernel below in 16-byte pieces, for bfloat16 with head sizes in eights.
+template <int NT>
+__global__ __launch_bounds__(NT) void qkv_rows_vec8_kernel(const bf16* __restrict__ qkv, const float* __restrict__ qw,
+                                                           const float* __restrict__ kw, float eps,
+                                                           const bf16* __restrict__ v_other, long long v_other_stride,
+                                                           float mix, const long long* __restrict__ slots,
+                                                           bf16* __restrict__ q_out, bf16* __restrict__ k_cache,
+                                                           bf16* __restrict__ v_cache, int page_size, int nq, int nkv, int d,
+                                                           int dv, int v_grouped) {
+  __shared__ float scratch[NT / kWave];
+  const int t = blockIdx.x;
+  const int nqd = nq * d, nkd = nkv * d, nvd = nkv * dv;
+  const bf16* row = qkv + (size_t)t * (nqd + nkd + nvd);
+  float invq = 1.f, invk = 1.f;
+  if (qw) {
+    float sq = 0.f, sk = 0.f;
+    for (int i = 8 * threadIdx.x; i < nqd + nkd; i += 8 * NT) {        // a piece lies in q or in k: both in eights
+      const bf16x8_t c = *reinterpret_cast<const bf16x8_t*>(row + i);
+      float a = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) a += to_float(c.v[e]) * to_float(c.v[e]);
+      if (i < nqd) sq += a;
+      else sk += a;
+    }
+    invq = rsqrtf(block_sum<NT / kWave>(sq, scratch) / (float)nqd + eps);
+    invk = rsqrtf(block_sum<NT / kWave>(sk, scratch) / (float)nkd + eps);
+  }
+  const long long slot = slots[t];
+  const size_t page = slot < 0 ? 0 : (size_t)(slot / page_size);
+  const int off = slot < 0 ? 0 : (int)(slot % page_size);
+  for (int i = 8 * threadIdx.x; i < nqd + nkd; i += 8 * NT) {
+    bf16x8_t c = *reinterpret_cast<const bf16x8_t*>(row + i);
+    const bool is_q = i < nqd;
+    if (qw) {
+      const float* wp = is_q ? qw + i : kw + (i - nqd);
+      const float4 w0 = load4(wp), w1 = load4(wp + 4);
+      const float ws[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+      const float inv = is_q ? invq : invk;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) c.v[e] = from_float<bf16>(to_float(c.v[e]) * inv * ws[e]);
+    }
+    if (is_q) {
+      *reinterpret_cast<bf16x8_t*>(q_out + (size_t)t * nqd + i) = c;
+    } else if (slot >= 0) {
+      const int ik = i - nqd, h = ik / d, cc = ik - h * d;
+      *reinterpret_cast<bf16x8_t*>(k_cache + ((page * nkv + h) * page_size + off) * d + cc) = c;
+    }
+  }
+  if (slot < 0) return;
+  const bf16* vo = v_other ? v_other + (size_t)t * v_other_stride : nullptr;
+  for (int i = 8 * threadIdx.x; i < nvd; i += 8 * NT) {
+    bf16x8_t c = *reinterpret_cast<const bf16x8_t*>(row + nqd + nkd + i);
+    if (vo) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) c.v[e] = from_float<bf16>((1.f - mix) * to_float(c.v[e]) + mix * to_float(vo[i + e]));
+    }
+    const int h = i / dv, cc = i - h * dv;
+    const size_t base = (page * nkv + h) * (size_t)page_size * dv;
+    if (v_grouped) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v_cache[base + ((size_t)(off >> 3) * dv + cc + e) * 8 + (off & 7)] = c.v[e];
+    } else {
+      *reinterpret_cast<bf16x8_t*>(v_cache + base + (size_t)off * dv + cc) = c;
+    }
   }
 }
 
@@ -787,8 +914,22 @@ int xi_rmsnorm_add(float* resid, const void* y, int y_dtype, int parts, const fl
   if (n_rows == 0) return 0;
   const size_t part_stride = (size_t)n_rows * H;
   constexpr int NT = 256;
-#define XI_RA(TY, TR) \
-  rmsnorm_add_kernel<TY, TR, NT><<<n_rows, NT, 0, stream>>>(resid, (const TY*)y, parts, part_stride, w, eps, (TR*)rows, H)
+  const bool vec = H % 4 == 0 && ((uintptr_t)resid | (uintptr_t)y | (uintptr_t)w | (uintptr_t)rows) % 16 == 0 &&
+                   (part_stride % 4 == 0 || parts == 1);
+  const bool few = vec && n_rows <= 256 && H <= 4 * 1024 * 2;       // few rows: 1024 threads a row (see xi_add_rmsnorm)
+  const bool many = vec && !few && H <= 4 * NT * 8;
+#define XI_RA(TY, TR)                                                                                                   \
+  do {                                                                                                                  \
+    if (few)                                                                                                            \
+      rmsnorm_add_vec_kernel<TY, TR, 1024, 2><<<n_rows, 1024, 0, stream>>>(resid, (const TY*)y, parts, part_stride, w,  \
+                                                                           eps, (TR*)rows, H);                          \
+    else if (many)                                                                                                      \
+      rmsnorm_add_vec_kernel<TY, TR, NT, 8><<<n_rows, NT, 0, stream>>>(resid, (const TY*)y, parts, part_stride, w, eps, \
+                                                                       (TR*)rows, H);                                   \
+    else                                                                                                                \
+      rmsnorm_add_kernel<TY, TR, NT><<<n_rows, NT, 0, stream>>>(resid, (const TY*)y, parts, part_stride, w, eps,        \
+                                                                (TR*)rows, H);                                          \
+  } while (0)
   if (y_dtype == kF32 && (rows == nullptr || rows_dtype == kF32)) XI_RA(float, float);
   else if (y_dtype == kF32 && rows_dtype == kBF16) XI_RA(float, bf16);
   else if (y_dtype == kBF16 && (rows == nullptr || rows_dtype == kBF16)) XI_RA(bf16, bf16);
@@ -807,7 +948,13 @@ int xi_act_mul(const void* gate_up, void* out, int dtype, int act, int n_tok, in
   size_t blocks = (total + 255) / 256;
   if (blocks > 65535u * 16u) blocks = 65535u * 16u;
 #define XI_AM(TT, A) act_mul_kernel<TT, A><<<(unsigned)blocks, 256, 0, stream>>>((const TT*)gate_up, (TT*)out, I, total)
-  if (dtype == kF32 && act == kSilu) XI_AM(float, kSilu);
+  if (dtype == kBF16 && I % 8 == 0 && ((uintptr_t)gate_up | (uintptr_t)out) % 16 == 0) {
+    const size_t total8 = total / 8;
+    size_t b8 = (total8 + 255) / 256;
+    if (b8 > 65535u * 16u) b8 = 65535u * 16u;
+    if (act == kSilu) act_mul_vec8_kernel<kSilu><<<(unsigned)b8, 256, 0, stream>>>((const bf16*)gate_up, (bf16*)out, I, total8);
+    else act_mul_vec8_kernel<kGeluTanh><<<(unsigned)b8, 256, 0, stream>>>((const bf16*)gate_up, (bf16*)out, I, total8);
+  } else if (dtype == kF32 && act == kSilu) XI_AM(float, kSilu);
   else if (dtype == kF32) XI_AM(float, kGeluTanh);
   else if (dtype == kBF16 && act == kSilu) XI_AM(bf16, kSilu);
   else if (dtype == kBF16) XI_AM(bf16, kGeluTanh);
@@ -829,7 +976,13 @@ int xi_qkv_rows(const void* qkv, int dtype, const float* qw, const float* kw, fl
   XI_CHECK(v_other == nullptr || v_other_stride >= (long long)nkv * dv, "qkv_rows: the other values' rows are too short");
   if (n_tok == 0) return 0;
   constexpr int NT = 256;
-  if (dtype == kF32)
+  if (dtype == kBF16 && d % 8 == 0 && dv % 8 == 0 && (v_other == nullptr || v_other_stride % 8 == 0) &&
+      ((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)v_other | (uintptr_t)qw |
+       (uintptr_t)kw) % 16 == 0)
+    qkv_rows_vec8_kernel<NT><<<n_tok, NT, 0, stream>>>((const bf16*)qkv, qw, kw, eps, (const bf16*)v_other, v_other_stride, mix,
+                                                       slots, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, page_size, nq, nkv,
+                                                       d, dv, v_grouped);
+  else if (dtype == kF32)
     qkv_rows_kernel<float, NT><<<n_tok, NT, 0, stream>>>((const float*)qkv, qw, kw, eps, (const float*)v_other, v_other_stride,
                                                          mix, slots, (float*)q_out, (float*)k_cache, (float*)v_cache,
                                                          page_size, nq, nkv, d, dv, v_grouped);

@@ -17,6 +17,7 @@
 
 namespace xi {
 
+struct alignas(16) Bf8 { bf16 v[8]; };
 constexpr int kRouteWaves = 4;
 constexpr int kMaxExperts = 1024;
 constexpr int kMaxTop = 64;
@@ -98,9 +99,27 @@ __global__ __launch_bounds__(kMoeWaves* kWave) void moe_gate_up_kernel(const T* 
     const T* g = wg + (size_t)f * H;
     const T* u = wg + (size_t)(F + f) * H;
     float ag = 0.f, au = 0.f;
-    for (int k = lane; k < H; k += kWave) {
-      ag = fmaf(to_float(g[k]), xs[k], ag);
-      au = fmaf(to_float(u[k]), xs[k], au);
+    if constexpr (sizeof(T) == 2) {
+      if (H % 8 == 0) {              // 16 bytes a lane and load; the order of a sum is still fixed by H alone
+        for (int k = 8 * lane; k < H; k += 8 * kWave) {
+          const Bf8 gv = *reinterpret_cast<const Bf8*>(g + k), uv = *reinterpret_cast<const Bf8*>(u + k);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            ag = fmaf(to_float(gv.v[e]), xs[k + e], ag);
+            au = fmaf(to_float(uv.v[e]), xs[k + e], au);
+          }
+        }
+      } else {
+        for (int k = lane; k < H; k += kWave) {
+          ag = fmaf(to_float(g[k]), xs[k], ag);
+          au = fmaf(to_float(u[k]), xs[k], au);
+        }
+      }
+    } else {
+      for (int k = lane; k < H; k += kWave) {
+        ag = fmaf(to_float(g[k]), xs[k], ag);
+        au = fmaf(to_float(u[k]), xs[k], au);
+      }
     }
     ag = wave_sum(ag);
     au = wave_sum(au);
@@ -124,7 +143,15 @@ __global__ __launch_bounds__(kMoeWaves* kWave) void moe_down_kernel(const T* __r
     for (int r = 0; r < top; ++r) {
       const T* w = wd + ((size_t)idx[(size_t)t * top + r] * H + n) * F;
       float acc = 0.f;
-      for (int f = lane; f < F; f += kWave) acc = fmaf(to_float(w[f]), ms[r * F + f], acc);
+      if (sizeof(T) == 2 && F % 8 == 0) {
+        for (int f = 8 * lane; f < F; f += 8 * kWave) {
+          const Bf8 wv = *reinterpret_cast<const Bf8*>(w + f);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc = fmaf(to_float(wv.v[e]), ms[r * F + f + e], acc);
+        }
+      } else {
+        for (int f = lane; f < F; f += kWave) acc = fmaf(to_float(w[f]), ms[r * F + f], acc);
+      }
       acc = wave_sum(acc);
       total += wt[(size_t)t * top + r] * acc;
     }

@@ -1,6 +1,6 @@
 // Routed experts for many tokens on the gfx950 matrix cores (bfloat16): the (token, chosen expert)
 // pairs are put in the order of their experts on the device, and each expert's rows go through its
-// weights in tiles, so a weight is read once per tile of up to 64 rows instead of once per pair.
+// weights in tiles, so a weight is read once per tile of up to 128 rows instead of once per pair.
 //
 //   moe_sort      pairs [T * top] -> `order` (slot -> pair), `slot_of` (pair -> slot), and the list of
 //                 tiles (expert, first slot, rows); one workgroup, nothing read on the host
@@ -145,6 +145,107 @@ __global__ __launch_bounds__(256) void moe_group_kernel(const bf16* __restrict__
     }
 }
 
+// The same product for tiles of up to 128 rows (experts with many rows): the rows' operand goes through LDS, read
+// from memory once a workgroup instead of once a wave (two buffers, one barrier a K step; a row of 32 k is padded
+// by 16 bytes against bank conflicts), the weights' operand stays with the wave that owns its features, and every
+// operand of a K step feeds 8 x NB products.  The next step's loads are in flight while this one is multiplied.
+template <bool GATED, int ACT>
+__global__ __launch_bounds__(256) void moe_group_lds_kernel(const bf16* __restrict__ A, const int* __restrict__ order, int top,
+                                                            const bf16* __restrict__ W, const int* __restrict__ tile_expert,
+                                                            const int* __restrict__ tile_row0,
+                                                            const int* __restrict__ tile_rows, const int* __restrict__ n_tiles,
+                                                            void* __restrict__ out, int N, int K) {
+  constexpr int MI = 8, BM = 128, LDA = 32 + 8;
+  __shared__ __align__(16) bf16 As[2][BM * LDA];
+  const int tile = blockIdx.x;
+  if (tile >= *n_tiles) return;
+  const int e = tile_expert[tile], row0 = tile_row0[tile], rows = tile_rows[tile];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, j = lane >> 4;
+  const int nw0 = blockIdx.y * 128 + wave * 32;
+  const bool owns = nw0 < N;                 // (a wave without features still copies rows and meets the barriers)
+  const bf16* agp[2];
+  int adst[2], ach[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int idx = tid + 256 * i, row = idx >> 2;
+    ach[i] = 8 * (idx & 3);
+    int slot = row0 + row;
+    slot = slot < row0 + rows ? slot : row0 + rows - 1;
+    const size_t arow = GATED ? (size_t)(order[slot] / top) : (size_t)slot;
+    agp[i] = A + arow * K + ach[i];
+    adst[i] = row * LDA + ach[i];
+  }
+  constexpr int NB = GATED ? 4 : 2;
+  const bf16* bp[NB];
+  const bf16* We = W + (size_t)e * (GATED ? 2 : 1) * N * K;
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    int col = nw0 + 16 * c + r;
+    col = col < N ? col : N - 1;
+    bp[c] = We + (size_t)col * K + 8 * j;
+    if (GATED) bp[2 + c] = We + (size_t)(N + col) * K + 8 * j;
+  }
+  mf32x4 acc[MI][NB];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int c = 0; c < NB; ++c) acc[i][c] = mf32x4{0.f, 0.f, 0.f, 0.f};
+  mbf16x8 an[2], b[NB], bn[NB];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) an[i] = ach[i] < K ? mld8(agp[i]) : mzero8();
+#pragma unroll
+  for (int c = 0; c < NB; ++c) b[c] = 8 * j < K ? mld8(bp[c]) : mzero8();
+#pragma unroll
+  for (int i = 0; i < 2; ++i) *reinterpret_cast<mbf16x8*>(&As[0][adst[i]]) = an[i];
+  __syncthreads();
+  int buf = 0;
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const bool next = k0 + 32 < K;
+    if (next) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) an[i] = k0 + 32 + ach[i] < K ? mld8(agp[i] + k0 + 32) : mzero8();
+#pragma unroll
+      for (int c = 0; c < NB; ++c) bn[c] = k0 + 32 + 8 * j < K ? mld8(bp[c] + k0 + 32) : mzero8();
+    }
+    if (owns) {
+      mbf16x8 a[MI];
+#pragma unroll
+      for (int i = 0; i < MI; ++i) a[i] = *reinterpret_cast<const mbf16x8*>(&As[buf][(16 * i + r) * LDA + 8 * j]);
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int c = 0; c < NB; ++c) acc[i][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[c], acc[i][c], 0, 0, 0);
+    }
+    if (next) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) *reinterpret_cast<mbf16x8*>(&As[buf ^ 1][adst[i]]) = an[i];
+#pragma unroll
+      for (int c = 0; c < NB; ++c) b[c] = bn[c];
+    }
+    __syncthreads();
+    buf ^= 1;
+  }
+  if (!owns) return;
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int row = 16 * i + 4 * j + v;
+      if (row >= rows) continue;
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const int col = nw0 + 16 * c + r;
+        if (col >= N) continue;
+        const size_t at = (size_t)(row0 + row) * N + col;
+        if (GATED)
+          reinterpret_cast<bf16*>(out)[at] = __float2bfloat16(moe_act_m<ACT>(acc[i][c][v]) * acc[i][GATED ? 2 + c : c][v]);
+        else
+          reinterpret_cast<float*>(out)[at] = acc[i][c][v];
+      }
+    }
+}
+
 __global__ void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ slot_of, const float* __restrict__ wt,
                                    float* __restrict__ out, int H, int top) {
   const int t = blockIdx.x;
@@ -167,7 +268,7 @@ int xi_moe_tiles_most(int P, int E, int bm) { return (P + bm - 1) / bm + E; }
 // idx int32 [P] (expert of every pair) -> order, slot_of int32 [P]; tile_* int32 [xi_moe_tiles_most]; n_tiles int32 [1].
 int xi_moe_sort(const int* idx, int P, int E, int bm, int* order, int* slot_of, int* tile_expert, int* tile_row0,
                 int* tile_rows, int* n_tiles, hipStream_t stream) {
-  XI_CHECK(P > 0 && E > 0 && E <= kSortExperts && (bm == 32 || bm == 64), "moe_sort: bad sizes pairs=%d experts=%d rows=%d", P, E, bm);
+  XI_CHECK(P > 0 && E > 0 && E <= kSortExperts && (bm == 32 || bm == 64 || bm == 128), "moe_sort: bad sizes pairs=%d experts=%d rows=%d", P, E, bm);
   moe_sort_kernel<<<1, kSortThreads, 0, stream>>>(idx, P, E, bm, order, slot_of, tile_expert, tile_row0, tile_rows, n_tiles);
   XI_LAUNCH_CHECK("moe_sort");
   return 0;
@@ -178,7 +279,7 @@ int xi_moe_sort(const int* idx, int P, int E, int bm, int* order, int* slot_of, 
 int xi_moe_group(const void* A, const int* order, int top, const void* W, const int* tile_expert, const int* tile_row0,
                  const int* tile_rows, const int* n_tiles, int tiles_most, void* out, int N, int K, int bm, int gated, int act,
                  hipStream_t stream) {
-  XI_CHECK(N > 0 && K > 0 && K % 8 == 0 && top > 0 && tiles_most > 0 && (bm == 32 || bm == 64),
+  XI_CHECK(N > 0 && K > 0 && K % 8 == 0 && top > 0 && tiles_most > 0 && (bm == 32 || bm == 64 || bm == 128),
            "moe_group: bad sizes N=%d K=%d (a multiple of 8) top=%d tiles=%d rows=%d", N, K, top, tiles_most, bm);
   XI_CHECK(act == 0 || act == 1, "moe_group: unknown activation %d", act);
   dim3 grid((unsigned)tiles_most, (unsigned)((N + 127) / 128));
@@ -186,7 +287,14 @@ int xi_moe_group(const void* A, const int* order, int top, const void* W, const 
 #define XI_MG(MI, G, ACT_)                                                                                            \
   moe_group_kernel<MI, G, ACT_><<<grid, 256, 0, stream>>>((const bf16*)A, order, top, (const bf16*)W, tile_expert,    \
                                                           tile_row0, tile_rows, n_tiles, out, N, K)
-  if (bm == 32) {
+  if (bm == 128) {
+    if (!gated) moe_group_lds_kernel<false, 0><<<grid, 256, 0, stream>>>((const bf16*)A, order, top, (const bf16*)W, tile_expert,
+                                                                         tile_row0, tile_rows, n_tiles, out, N, K);
+    else if (act == 0) moe_group_lds_kernel<true, 0><<<grid, 256, 0, stream>>>((const bf16*)A, order, top, (const bf16*)W,
+                                                                               tile_expert, tile_row0, tile_rows, n_tiles, out, N, K);
+    else moe_group_lds_kernel<true, 1><<<grid, 256, 0, stream>>>((const bf16*)A, order, top, (const bf16*)W, tile_expert,
+                                                                 tile_row0, tile_rows, n_tiles, out, N, K);
+  } else if (bm == 32) {
     if (!gated) XI_MG(2, false, 0);
     else if (act == 0) XI_MG(2, true, 0);
     else XI_MG(2, true, 1);

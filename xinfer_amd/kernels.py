@@ -325,7 +325,7 @@ def moe_grouped_takes(T: int, top: int, E: int, H: int, F: int, dtype: torch.dty
 
 
 def moe_experts(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx: torch.Tensor, wt: torch.Tensor,
-                act: str = "silu", grouped: Optional[bool] = None) -> torch.Tensor:
+                act: str = "silu", grouped: Optional[bool] = None, tile_rows: Optional[int] = None) -> torch.Tensor:
     """sum over a token's chosen experts e (in the order of `idx`) of wt * down[e] @ (act(gate[e] @ x) * (up[e] @ x)):
     gate_up [E, 2F, H] (gate rows first), down [E, H, F], idx int32 / wt float32 [T, top].  Float32 [T, H].
     One (token, expert) pair at a time, every sum in an order fixed by the sizes: the form of the
@@ -354,7 +354,11 @@ def moe_experts(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx:
         if not moe_grouped_takes(T, top, E, H, F, x.dtype, force=True):
             raise KernelError(f"moe_experts: the grouped form takes bfloat16 and sizes in eights, not {x.dtype} H={H} F={F}")
         P = T * top
-        bm = 64 if P >= 48 * E else 32               # rows of a tile: 64 where most experts fill them
+        if tile_rows is None:                        # rows of a tile: as many as most experts fill
+            tile_rows = 128 if P >= 96 * E else 64 if P >= 48 * E else 32
+        bm = int(tile_rows)
+        if bm not in (32, 64, 128):
+            raise KernelError("moe_experts: tiles of 32, 64 or 128 rows")
         most = int(lib().xi_moe_tiles_most(P, E, bm))
         ints = torch.empty((2 * P + 3 * most + 1,), dtype=torch.int32, device=x.device)
         order, slot_of = ints[:P], ints[P:2 * P]
