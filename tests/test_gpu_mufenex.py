@@ -346,6 +346,8 @@ def test_experts_grouped_on_the_matrix_cores(E, top, H, F, T):
     one = kernels.moe_experts(x.to(DEV), gu, dn, gi, gw, "silu", grouped=False)
     got = kernels.moe_experts(x.to(DEV), gu, dn, gi, gw, "silu", grouped=True)
     assert (got - one).abs().max() <= 0.02 * one.abs().max()
+    lib_out = kernels.moe_experts_library(x.to(DEV), gu, dn, gi, gw, "silu")          # the vendor library's products an expert
+    assert (lib_out - one).abs().max() <= 0.02 * one.abs().max()
     for rows in (32, 64, 128):                   # every tile height gives a row the same sums
         again = kernels.moe_experts(x.to(DEV), gu, dn, gi, gw, "silu", grouped=True, tile_rows=rows)
         assert torch.equal(again, got), f"tiles of {rows} rows"

@@ -34,9 +34,20 @@ __global__ __launch_bounds__(kRouteWaves* kWave) void moe_route_kernel(const T* 
   const T* xr = x + (size_t)t * H;
   for (int e = wave; e < E; e += kRouteWaves) {
     const float* w = wr + (size_t)e * H;
-    float acc = 0.f;
-    for (int k = lane; k < H; k += kWave) acc = fmaf(to_float(xr[k]), w[k], acc);
-    acc = wave_sum(acc);
+    // four chains a lane, so that four rounds of loads are in flight; the order is fixed by H alone
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int k = lane;
+    for (; k + 3 * kWave < H; k += 4 * kWave) {
+      const float x0 = to_float(xr[k]), x1 = to_float(xr[k + kWave]), x2 = to_float(xr[k + 2 * kWave]),
+                  x3 = to_float(xr[k + 3 * kWave]);
+      const float w0 = w[k], w1 = w[k + kWave], w2 = w[k + 2 * kWave], w3 = w[k + 3 * kWave];
+      a0 = fmaf(x0, w0, a0);
+      a1 = fmaf(x1, w1, a1);
+      a2 = fmaf(x2, w2, a2);
+      a3 = fmaf(x3, w3, a3);
+    }
+    for (; k < H; k += kWave) a0 = fmaf(to_float(xr[k]), w[k], a0);
+    float acc = wave_sum((a0 + a1) + (a2 + a3));
     if (lane == 0) z[e] = acc + (br ? br[e] : 0.f);
   }
   __syncthreads();

@@ -324,6 +324,47 @@ def moe_grouped_takes(T: int, top: int, E: int, H: int, F: int, dtype: torch.dty
     return force or (MOE_GROUPED and T * top > E)
 
 
+MOE_LIBRARY_ROWS = 64     # rows an expert on average from which a step of portions takes the vendor library's products
+
+
+def moe_experts_library(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx: torch.Tensor, wt: torch.Tensor,
+                        act: str = "silu") -> torch.Tensor:
+    """`moe_experts` for steps of many tokens in bfloat16: the pairs sorted by expert on the device, the rows
+    gathered in that order, and one plain product of the vendor library an expert and projection (as the
+    dense feed-forward's products of many rows go to the library); the hand-written kernels do the sort,
+    the activation and the combine.  Reads the experts' row counts on the host: for steps that bring
+    portions, which are never recorded into a graph."""
+    _dev(x, gate_up, down, idx, wt)
+    T, H = x.shape
+    E, F2, _ = gate_up.shape
+    F, top = F2 // 2, int(idx.shape[1])
+    if x.dtype != torch.bfloat16 or gate_up.dtype != torch.bfloat16 or down.dtype != torch.bfloat16:
+        raise KernelError("moe_experts_library: operands must be bfloat16")
+    if gate_up.shape != (E, 2 * F, H) or down.shape != (E, H, F) or idx.shape != (T, top) or wt.shape != (T, top):
+        raise KernelError("moe_experts_library: x [T, H], gate_up [E, 2F, H], down [E, H, F], idx and weights [T, top]")
+    _want(idx, torch.int32, "moe_experts_library: idx")
+    _want(wt, torch.float32, "moe_experts_library: weights")
+    P = T * top
+    most = int(lib().xi_moe_tiles_most(P, E, 128))
+    ints = torch.empty((2 * P + 3 * most + 1,), dtype=torch.int32, device=x.device)
+    order, slot_of = ints[:P], ints[P:2 * P]
+    _ok(lib().xi_moe_sort(_p(idx), P, E, 128, _p(order), _p(slot_of), _p(ints[2 * P:2 * P + most]),
+                          _p(ints[2 * P + most:2 * P + 2 * most]), _p(ints[2 * P + 2 * most:2 * P + 3 * most]),
+                          _p(ints[2 * P + 3 * most:]), _stream()))
+    counts = torch.bincount(idx.reshape(-1), minlength=E).tolist()          # the one read on the host
+    rows = x.index_select(0, torch.div(order, top, rounding_mode="floor"))
+    y = torch.empty((P, H), dtype=torch.float32, device=x.device)
+    at = 0
+    for e, n in enumerate(counts[:E]):
+        if n:
+            mid = act_mul(torch.nn.functional.linear(rows[at:at + n], gate_up[e]), act)
+            torch.mm(mid, down[e].t(), out_dtype=torch.float32, out=y[at:at + n])
+            at += n
+    out = torch.empty((T, H), dtype=torch.float32, device=x.device)
+    _ok(lib().xi_moe_combine(_p(y), _p(slot_of), _p(wt), _p(out), T, H, top, _stream()))
+    return out
+
+
 def moe_experts(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx: torch.Tensor, wt: torch.Tensor,
                 act: str = "silu", grouped: Optional[bool] = None, tile_rows: Optional[int] = None) -> torch.Tensor:
     """sum over a token's chosen experts e (in the order of `idx`) of wt * down[e] @ (act(gate[e] @ x) * (up[e] @ x)):

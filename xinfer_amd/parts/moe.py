@@ -4,8 +4,8 @@ z = W_router x (+ b) in float32; each token takes the `top` experts with the lar
 the softmax over the chosen logits only; an expert is a gated feed-forward without biases,
 down(act(gate x) * (up x)); the result is the weighted sum of the chosen experts' outputs, in
 float32.  The experts' weights are stacked at load: gate and up [E, 2F, H] (gate rows first), down
-[E, H, F].  Nothing of a step is read on the host: the router's choice stays on the device and the
-experts' kernels find their rows from it, so decode steps can be recorded.
+[E, H, F].  In steps of single tokens nothing is read on the host: the router's choice stays on the
+device and the experts' kernels find their rows from it, so decode steps can be recorded.
 
 Tensor names under the part's prefix (`names` of the spec replaces any of them): `router`,
 `router_bias`, and per expert i `expert{i}.gate`, `expert{i}.up`, `expert{i}.down`, in which "{i}" is
@@ -26,6 +26,7 @@ from .base import FeedForward, StepContext, register_feed_forward
 @register_feed_forward("routed_experts")
 class RoutedExperts(FeedForward):
     graph_safe = True
+    LIBRARY = True       # False: the hand-written kernels for every step
     NAMES = {"router": "router.weight", "router_bias": "router.bias", "gate": "experts.{i}.gate_proj.weight",
              "up": "experts.{i}.up_proj.weight", "down": "experts.{i}.down_proj.weight"}
 
@@ -78,4 +79,9 @@ class RoutedExperts(FeedForward):
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         idx, wt = kernels.moe_route(x, self.router_w, self.router_b, self.top)
+        # a step that brings portions is never recorded: with many rows an expert it may read the experts' row
+        # counts on the host and hand each expert's rows to the vendor library, as the dense products of many rows go
+        if (ctx.max_q_len > 1 and x.dtype == torch.bfloat16 and self.LIBRARY
+                and x.shape[0] * self.top >= kernels.MOE_LIBRARY_ROWS * self.experts):
+            return kernels.moe_experts_library(x, self.gate_up, self.down, idx, wt, self.activation)
         return kernels.moe_experts(x, self.gate_up, self.down, idx, wt, self.activation)
