@@ -7,6 +7,8 @@ Q: the values that other models happen to make equal or 1: value size = key size
 and as many kv heads as heads, one chosen expert, no embedding scale, no soft cap on the logits,
 a layer that blends no values before the ones that do (so the first blending layer is not
 layer 0), a width that is no multiple of 8.
+S: nothing blended anywhere, no cap on any score, windows of 1 and 2 keys and one wider than any request, all
+experts chosen, a first layer without feed-forward, head sizes in eights that are no multiple of 16.
 R: real-looking head sizes (64 and 128) with few layers, for the matrix-core kernels.
 
 Random weights would leave the router's choice to close calls (bfloat16 rounds the stream, and two
@@ -58,6 +60,13 @@ MODELS = {
             _layer(_mixer(5, 1, 32, 80, 0.18, softcap=15.0, window=17), _moe(40, 7, 3)),
             _layer(_mixer(1, 1, 48, 80, 0.15, softcap=50.0, window=9), {"kind": "dense", "ff": 56})]},
         seed=12, linear_std=0.1, norm_std=0.2, page_size=8),
+    "S": dict(
+        config={"architecture": "Mufenex", "vocab": 190, "width": 72, "embedding": {"scale": 1.5}, "norm": {"eps": 1e-6},
+                "logit_softcap": 20.0, "layers": [
+                    _layer(_mixer(6, 3, 24, 40, 0.2, window=1, v_mix=False), None),
+                    _layer(_mixer(3, 3, 8, 8, 0.35, window=200, v_mix=False), _moe(16, 3, 3)),
+                    _layer(_mixer(2, 2, 40, 24, 0.16, window=2, v_mix=False), {"kind": "dense", "ff": 40})]},
+        seed=14, linear_std=0.1, norm_std=0.15, page_size=8),
     "R": dict(
         config={"architecture": "Mufenex", "vocab": 409, "width": 512, "embedding": {"scale": 2.0},
                 "norm": {"eps": 1e-6}, "logit_softcap": 30.0, "layers": [

@@ -359,7 +359,8 @@ def test_experts_grouped_on_the_matrix_cores(E, top, H, F, T):
 
 
 # ---- whole models ---------------------------------------------------------------------------------
-LENGTHS = {"P": [1, 2, 12, 13, 33, 77, 130], "Q": [3, 9, 10, 18, 64, 101], "R": [5, 101, 330, 64, 301]}
+LENGTHS = {"P": [1, 2, 12, 13, 33, 77, 130], "Q": [3, 9, 10, 18, 64, 101], "S": [1, 2, 3, 50, 90],
+           "R": [5, 101, 330, 64, 301]}
 
 
 def _requests(name):
@@ -485,6 +486,10 @@ def test_greedy_generation_through_the_engine(dtype, dirs):
 
 def test_command_line_runs_the_model(dirs, capsys):
     from xinfer_amd import cli
+    # the engine plans its own pages (three cache groups) where none are given
+    rc = cli.main(["--w", dirs("P"), "--prompt-ids", "1,2,3,4,5,6,7,8,9", "--max-tokens", "4", "--max-model-len", "256",
+                   "--temperature", "0", "--ignore-eos", "--page-size", "16", "--max-num-seqs", "4", "--dtype", "bf16"])
+    assert rc == 0 and "Decoded tokens: 4 in" in capsys.readouterr().out
     rc = cli.main(["--w", dirs("Q"), "--prompt-ids", "1,2,3|4,5,6,7", "--max-tokens", "5", "--max-model-len", "64",
                    "--temperature", "0", "--ignore-eos", "--page-size", "8", "--num-pages", "16", "--dtype", "f32"])
     out = capsys.readouterr().out
