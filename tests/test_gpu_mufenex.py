@@ -92,6 +92,19 @@ def test_activations_times_up():
         assert (got - want).abs().max() < 0.02 * want.abs().max()
 
 
+@pytest.mark.parametrize("M", [2, 8, 33])
+def test_gate_up_product_with_the_activation_inside(M):
+    """The tiled gate/up product of decode steps applies the tanh form of gelu as it applies silu."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(M)
+    x = torch.randn(M, 192, generator=g).to(torch.bfloat16)
+    w = (torch.randn(2 * 104, 192, generator=g) * 0.2).to(torch.bfloat16)
+    for act, f in (("gelu_tanh", plain.gelu_tanh), ("silu", plain.silu)):
+        want = f(x.double() @ w[:104].double().T) * (x.double() @ w[104:].double().T)
+        got = kernels.linear_mid_gated(x.to(DEV), w.to(DEV), act=act).cpu().double()
+        assert (got - want).abs().max() < 0.02 * want.abs().max()
+
+
 def _pools(L, G, d, dv, page, dtype, grouped, seed=0):
     """Empty K and V pools with more pages than L tokens need, and a block table of shuffled pages."""
     n_pages = -(-L // page)

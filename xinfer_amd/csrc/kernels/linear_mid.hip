@@ -58,6 +58,7 @@ struct MidFold {
   int parts;
   float eps;
   float inv_h;          // 1 / length of the normed rows
+  int act = 0;          // gated form: 0 silu(gate) * up, 1 the tanh form of gelu
 };
 
 // D: tiles whose loads are in flight.  FULL: up to 128 rows of x, the four waves take a quarter
@@ -232,7 +233,9 @@ __global__ __launch_bounds__(256, 1) void linear_mid_kernel(const bf16* __restri
         for (int i = 0; i < 4; ++i)
           if (f + i <= n_last) {
             const float g = acc[ti][tj][i] * inv, u = acc[ti + TG][tj][i] * inv;
-            dst[i] = from_float<bf16>(g / (1.f + __expf(-g)) * u);
+            const float a = fold.act == 0 ? g / (1.f + __expf(-g))
+                                          : 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+            dst[i] = from_float<bf16>(a * u);
           }
       }
     }
@@ -360,11 +363,12 @@ int xi_linear_mid(const void* x, const void* w, float* y, int M, int N, int K, i
   return 0;
 }
 
-// y [M, N] bfloat16 = silu(x @ gate^T) * (x @ up^T) with w = [gate; up] [2N, K], M <= 128.
+// y [M, N] bfloat16 = act(x @ gate^T) * (x @ up^T) with w = [gate; up] [2N, K], M <= 128; act 0: silu, 1: gelu (tanh form).
 // ss (or null): x is the first half of a folded RMSNorm, ss [M, parts] float32 the parts of its
 // rows' sums of squares (M <= 16, parts <= 512): rows are scaled by rsqrt(sum / K + eps).
 int xi_linear_mid_gated(const void* x, const void* w, void* y, int M, int N, int K, const float* ss, int parts,
-                        float eps, int rotate, int features, hipStream_t stream) {
+                        float eps, int rotate, int features, int act, hipStream_t stream) {
+  XI_CHECK(act == 0 || act == 1, "linear_mid_gated: unknown activation %d", act);
   XI_CHECK(M >= 1 && M <= kMidRows, "linear_mid_gated: M=%d must be 1..%d", M, kMidRows);
   XI_CHECK(N >= 1 && K >= kMidK && K % kMidK == 0, "linear_mid_gated: N=%d, K=%d (a multiple of %d) are not taken", N,
            K, kMidK);
@@ -376,7 +380,7 @@ int xi_linear_mid_gated(const void* x, const void* w, void* y, int M, int N, int
   const long long wgs = (N + R - 1) / R;
   XI_CHECK(R >= 1 && R <= 128 && wgs < (1ll << 31), "linear_mid_gated: %d features per workgroup", R);
   XI_CHECK(R <= 64 || (M <= 64 && ss == nullptr), "linear_mid_gated: %d features per workgroup are taken up to 64 rows, without a folded norm", R);
-  const MidFold fold{ss, parts, eps, 1.f / (float)K};
+  const MidFold fold{ss, parts, eps, 1.f / (float)K, act};
   if (R > 64) {
 #define XI_MIDW(TJ)                                                                                                     \
   do {                                                                                                                  \

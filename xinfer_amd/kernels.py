@@ -1140,8 +1140,8 @@ def gated_uses_mid(M: int, w: torch.Tensor) -> bool:
 
 
 def linear_mid_gated(x: torch.Tensor, w: torch.Tensor, ss: Optional[torch.Tensor] = None, eps: float = 0.0,
-                     features: Optional[int] = None) -> torch.Tensor:
-    """silu(x @ gate^T) * (x @ up^T) in bfloat16 for w = [gate; up] [2N, K] and up to MID_GATED_ROWS
+                     features: Optional[int] = None, act: str = "silu") -> torch.Tensor:
+    """act(x @ gate^T) * (x @ up^T), act silu unless given (`ACTIVATIONS`), in bfloat16 for w = [gate; up] [2N, K] and up to MID_GATED_ROWS
     rows with the tiled kernel: one pass over w whatever the number of rows.  `ss` [M, parts]
     float32 (up to FOLD_ROWS rows): x is the first half of a folded RMSNorm (`linear_fold_out`)
     and the rows of the products are multiplied by rsqrt(sum(ss[row]) / K + eps) first.
@@ -1165,7 +1165,7 @@ def linear_mid_gated(x: torch.Tensor, w: torch.Tensor, ss: Optional[torch.Tensor
         parts = int(ss.shape[1])
     y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
     _ok(lib().xi_linear_mid_gated(_p(x), _p(w), _p(y), M, N, K, _p(ss), parts, ctypes.c_float(eps), int(MID_GATED_ROTATE),
-                                  int(features if features is not None else MID_GATED_FEATURES), _stream()))
+                                  int(features if features is not None else MID_GATED_FEATURES), ACTIVATIONS[act], _stream()))
     return y
 
 

@@ -29,13 +29,13 @@ class Linear:
         self.out_features, self.in_features = weight.shape
 
     def __call__(self, x, out_dtype: Optional[torch.dtype] = None, skinny_rows: Optional[int] = None,
-                 allow_split: bool = False, sink: Optional[NormSink] = None, gated: bool = False):
+                 allow_split: bool = False, sink: Optional[NormSink] = None, gated: bool = False, act: str = "silu"):
         """`x`: rows, or a `Folded` (the norm before this product is half done: this product
         finishes it).  `sink`: the norm after this product may be folded: if the sizes allow
         (bfloat16, up to `kernels.FOLD_ROWS` rows) the result is added into the stream here and a
         `Folded` comes back instead of rows.  `gated`: the weight is [gate; up] and the result
-        silu(gate) * up, where the fused kernel takes the sizes (else None: the caller does it
-        in two steps).
+        act(gate) * up (`act`: silu, or the tanh form of gelu where the fused kernel has it), where the
+        fused kernel takes the sizes (else None: the caller does it in two steps).
         `allow_split`: the caller hands the result to a norm, which also takes a stack
         [P, T, out] of float32 partial sums; few rows and a narrow output then come back so.
         A workgroup of the split product takes more rows of the weight per read of x, which
@@ -43,6 +43,8 @@ class Linear:
         if skinny_rows is None:
             skinny_rows = kernels.SKINNY_ROWS
         w = self.weight
+        if isinstance(x, Folded) and gated and act != "silu":
+            x = x.rows(torch.bfloat16 if w.dtype == torch.bfloat16 else torch.float32)      # the folded products apply silu
         if isinstance(x, Folded):
             if w.dtype == torch.bfloat16 and x.xg.shape[1] % 8 == 0 and (not gated or out_dtype in (None, torch.bfloat16)):
                 if gated and kernels.gated_uses_mid(x.xg.shape[0], w):
@@ -53,7 +55,9 @@ class Linear:
             x = x.rows(torch.bfloat16 if w.dtype == torch.bfloat16 else torch.float32)
         if gated:
             if x.dtype == torch.bfloat16 and x.dim() == 2 and kernels.gated_uses_mid(x.shape[0], w):
-                return kernels.linear_mid_gated(x, w)                 # gate, up and silu*mul in one pass
+                return kernels.linear_mid_gated(x, w, act=act)        # gate, up and act*mul in one pass
+            if act != "silu":
+                return None                                           # the streaming kernel's gated form applies silu
             if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
                     and 0 < x.shape[0] <= kernels.SKINNY_GATED_ROWS and x.shape[1] % 8 == 0):
                 return kernels.linear_skinny(x, w, gated=True)        # the same with the streaming kernel

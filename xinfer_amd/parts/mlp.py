@@ -60,10 +60,9 @@ class GatedMLP(FeedForward):
 
     def forward(self, x, ctx: StepContext, sink=None):
         """`x`: rows or a `Folded`; `sink`: see `Part.takes_sink`."""
-        if self.activation != "silu":        # the fused products apply silu; other activations take two steps
+        m = self.gate_up(x, out_dtype=self.dtype, gated=True, act=self.activation)    # gate, up and act*mul in one pass
+        if m is None and self.activation != "silu":
             m = kernels.act_mul(self.gate_up(x, out_dtype=self.dtype), self.activation)
-            return self.down(m, out_dtype=self.dtype, allow_split=True, sink=sink)
-        m = self.gate_up(x, out_dtype=self.dtype, gated=True)         # gate, up and silu*mul in one pass
-        if m is None:
+        elif m is None:
             m = kernels.silu_mul(self.gate_up(x, out_dtype=self.dtype))
         return self.down(m, out_dtype=self.dtype, allow_split=True, sink=sink)   # the next norm adds the parts
