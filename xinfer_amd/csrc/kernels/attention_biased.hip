@@ -371,6 +371,30 @@ __global__ __launch_bounds__(64) void attn_biased_combine_kernel(const float* __
                                                                  int max_splits, int nq, int dv) {
   const int head = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
   const size_t base = ((size_t)t * nq + head) * max_splits;
+  __shared__ float f_s[64];
+  if (max_splits <= 64) {          // a slice a lane: one round of loads for the weights, one for the sums
+    float ms = -INFINITY, ls = 0.f;
+    if (lane < max_splits) {
+      const float2 ml = *reinterpret_cast<const float2*>(part_ml + (base + lane) * 2);
+      ms = ml.x;
+      ls = ml.y;
+    }
+    const float mm = wave_max(ms);
+    const float f = ms > -INFINITY ? __builtin_amdgcn_exp2f(ms - mm) : 0.f;
+    const float inv = 1.f / wave_sum(ls * f);
+    f_s[lane] = f;
+    __syncthreads();
+    for (int i = lane; i < dv; i += 64) {
+      float o = 0.f;
+#pragma unroll 4
+      for (int s2 = 0; s2 < max_splits; ++s2) {
+        const float fs = f_s[s2];
+        if (fs > 0.f) o += part_o[(base + s2) * dv + i] * fs;
+      }
+      out[((size_t)t * nq + head) * dv + i] = __float2bfloat16(o * inv);
+    }
+    return;
+  }
   float mm = -INFINITY;
   for (int s2 = 0; s2 < max_splits; ++s2) mm = fmaxf(mm, part_ml[(base + s2) * 2]);
   float ll = 0.f;

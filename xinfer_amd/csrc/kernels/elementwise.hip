@@ -485,12 +485,19 @@ __global__ void embed_sinusoid_kernel(const T* __restrict__ table, const int* __
   const T* row = table + (size_t)ids[t] * H;
   const float p = (float)positions[t];
   float* o = out + (size_t)t * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    const float ang = p * freq[i >> 1];
-    const float pe = (i & 1) ? cosf(ang) : sinf(ang);
-    const float v = to_float(row[i]) * scale + pe;
-    o[i] = v;
-    if (rows) rows[(size_t)t * H + i] = from_float<TR>(v);
+  for (int pair = threadIdx.x; 2 * pair < H; pair += blockDim.x) {      // a thread an angle: its sine and its cosine
+    const float ang = p * freq[pair];
+    float sn, cs;
+    sincosf(ang, &sn, &cs);
+    const int i = 2 * pair;
+    const float v0 = to_float(row[i]) * scale + sn;
+    o[i] = v0;
+    if (rows) rows[(size_t)t * H + i] = from_float<TR>(v0);
+    if (i + 1 < H) {
+      const float v1 = to_float(row[i + 1]) * scale + cs;
+      o[i + 1] = v1;
+      if (rows) rows[(size_t)t * H + i + 1] = from_float<TR>(v1);
+    }
   }
 }
 
@@ -895,8 +902,9 @@ int xi_embed_sinusoid(const void* table, int dtype, const int* ids, const int* p
                       void* rows, int rows_dtype, int n_tok, int H, float scale, hipStream_t stream) {
   XI_CHECK(n_tok >= 0 && H > 0, "embed_sinusoid: bad sizes T=%d H=%d", n_tok, H);
   if (n_tok == 0) return 0;
+  const int nt = H >= 2048 ? 1024 : (H >= 512 ? 256 : 64);        // about a pair a thread
 #define XI_ES(TT, TR) \
-  embed_sinusoid_kernel<TT, TR><<<n_tok, 256, 0, stream>>>((const TT*)table, ids, positions, freq, out, (TR*)rows, H, scale)
+  embed_sinusoid_kernel<TT, TR><<<n_tok, nt, 0, stream>>>((const TT*)table, ids, positions, freq, out, (TR*)rows, H, scale)
   if (dtype == kF32 && (rows == nullptr || rows_dtype == kF32)) XI_ES(float, float);
   else if (dtype == kBF16 && (rows == nullptr || rows_dtype == kBF16)) XI_ES(bf16, bf16);
   else if (dtype == kBF16 && rows_dtype == kF32) XI_ES(bf16, float);
