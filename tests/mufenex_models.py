@@ -9,6 +9,8 @@ a layer that blends no values before the ones that do (so the first blending lay
 layer 0), a width that is no multiple of 8.
 S: nothing blended anywhere, no cap on any score, windows of 1 and 2 keys and one wider than any request, all
 experts chosen, a first layer without feed-forward, head sizes in eights that are no multiple of 16.
+O: sizes in no kernel's favourite multiples (width 50, heads of 12, 20 and 10, 18 and 34 hidden features): every
+vectorized form steps aside for its plain one, in bfloat16 too.
 R: real-looking head sizes (64 and 128) with few layers, for the matrix-core kernels.
 
 Random weights would leave the router's choice to close calls (bfloat16 rounds the stream, and two
@@ -67,6 +69,12 @@ MODELS = {
                     _layer(_mixer(3, 3, 8, 8, 0.35, window=200, v_mix=False), _moe(16, 3, 3)),
                     _layer(_mixer(2, 2, 40, 24, 0.16, window=2, v_mix=False), {"kind": "dense", "ff": 40})]},
         seed=14, linear_std=0.1, norm_std=0.15, page_size=8),
+    "O": dict(
+        config={"architecture": "Mufenex", "vocab": 131, "width": 50, "embedding": {"scale": 0.9}, "norm": {"eps": 1e-5},
+                "logit_softcap": 12.0, "layers": [
+                    _layer(_mixer(3, 1, 12, 20, 0.3, softcap=25.0, window=7), _moe(18, 4, 2)),
+                    _layer(_mixer(2, 2, 20, 10, 0.22, softcap=25.0, window=30), {"kind": "dense", "ff": 34})]},
+        seed=15, linear_std=0.1, norm_std=0.1, page_size=8),
     "R": dict(
         config={"architecture": "Mufenex", "vocab": 409, "width": 512, "embedding": {"scale": 2.0},
                 "norm": {"eps": 1e-6}, "logit_softcap": 30.0, "layers": [

@@ -372,7 +372,7 @@ def test_experts_grouped_on_the_matrix_cores(E, top, H, F, T):
 
 
 # ---- whole models ---------------------------------------------------------------------------------
-LENGTHS = {"P": [1, 2, 12, 13, 33, 77, 130], "Q": [3, 9, 10, 18, 64, 101], "S": [1, 2, 3, 50, 90],
+LENGTHS = {"P": [1, 2, 12, 13, 33, 77, 130], "Q": [3, 9, 10, 18, 64, 101], "S": [1, 2, 3, 50, 90], "O": [1, 7, 8, 40, 75],
            "R": [5, 101, 330, 64, 301]}
 
 
