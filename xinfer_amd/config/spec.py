@@ -41,6 +41,7 @@ class LayerSpec:
     norms: Mapping[str, PartSpec]
     mixer_name: str = "self_attn"
     feed_forward_name: str = "mlp"
+    block_params: Mapping[str, Any] = field(default_factory=dict)    # constants of the arrangement itself
 
     def norm_items(self, count: int):
         """The first `count` norms as (tensor name under the prefix, spec), in running order."""
@@ -55,9 +56,13 @@ class LayerSpec:
 class ScheduleEntry:
     """One step of the run order.  `layer` indexes `ModelSpec.layers`; a layer may be
     named more than once.  `cache_of` makes this run read (and not write) the cache
-    that another layer's run owns; None means the layer's own."""
+    that another layer's run owns; None means the layer's own.  `cache_id` gives this run a
+    cache and state of its own under that number, whatever layer's weights it runs with (a
+    layer that is run again with the same tensors, as a layer of its own: ids and the indices
+    of layers that own a cache share one numbering, so an id is no such layer's index)."""
     layer: int
     cache_of: Optional[int] = None
+    cache_id: Optional[int] = None
 
 
 @dataclass(frozen=True)

@@ -80,7 +80,7 @@ __global__ void softcap_kernel(float* __restrict__ x, size_t n, float cap) {
 template <typename TY, typename TO, int NT>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TY* __restrict__ y, int parts, size_t part_stride,
                                    const float* __restrict__ w, float eps, TO* __restrict__ out,
-                                   const int* __restrict__ rows, int H) {
+                                   const int* __restrict__ rows, int H, float ys) {
   __shared__ float scratch[NT / kWave];
   const int r = blockIdx.x;
   const int row = rows ? rows[r] : r;
@@ -93,7 +93,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TY* __restri
   for (int i = threadIdx.x; i < H; i += NT) {
     float s = x[i];
     if (yr)
-      for (int p = 0; p < parts; ++p) s += to_float(yr[p * part_stride + i]);
+      for (int p = 0; p < parts; ++p) s = fmaf(ys, to_float(yr[p * part_stride + i]), s);
     ss += s * s;
   }
   const float total = block_sum<NT / kWave>(ss, scratch);
@@ -101,7 +101,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TY* __restri
   for (int i = threadIdx.x; i < H; i += NT) {
     float s = x[i];
     if (yr) {
-      for (int p = 0; p < parts; ++p) s += to_float(yr[p * part_stride + i]);
+      for (int p = 0; p < parts; ++p) s = fmaf(ys, to_float(yr[p * part_stride + i]), s);
       if (!rows) x[i] = s;
     }
     o[i] = from_float<TO>(s * inv * w[i]);
@@ -133,7 +133,7 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_vec_kernel(float* __restrict__
                                                              int parts, size_t part_stride,
                                                              const float* __restrict__ w, float eps,
                                                              TO* __restrict__ out, const int* __restrict__ rows,
-                                                             int H) {
+                                                             int H, float ys) {
   __shared__ float scratch[NT / kWave];
   const int r = blockIdx.x;
   const int row = rows ? rows[r] : r;
@@ -158,10 +158,10 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_vec_kernel(float* __restrict__
 #pragma unroll
           for (int p = 0; p < PB; ++p)
             if (p0 + p < parts) {
-              s[v].x += yy[p].x;
-              s[v].y += yy[p].y;
-              s[v].z += yy[p].z;
-              s[v].w += yy[p].w;
+              s[v].x = fmaf(ys, yy[p].x, s[v].x);      // ys = 1: the plain sum, bit for bit
+              s[v].y = fmaf(ys, yy[p].y, s[v].y);
+              s[v].z = fmaf(ys, yy[p].z, s[v].z);
+              s[v].w = fmaf(ys, yy[p].w, s[v].w);
             }
         }
       }
@@ -623,9 +623,13 @@ __global__ __launch_bounds__(NT) void qkv_rows_vec8_kernel(const bf16* __restric
                                                            float mix, const long long* __restrict__ slots,
                                                            bf16* __restrict__ q_out, bf16* __restrict__ k_cache,
                                                            bf16* __restrict__ v_cache, int page_size, int nq, int nkv, int d,
-                                                           int dv, int v_grouped) {
+                                                           int dv, int v_grouped, const float* __restrict__ cos_t,
+                                                           const float* __restrict__ sin_t, int rot,
+                                                           const int* __restrict__ positions) {
   __shared__ float scratch[NT / kWave];
   const int t = blockIdx.x;
+  const int half = rot / 2;
+  const size_t trow = rot ? (size_t)positions[t] * half : 0;
   const int nqd = nq * d, nkd = nkv * d, nvd = nkv * dv;
   const bf16* row = qkv + (size_t)t * (nqd + nkd + nvd);
   float invq = 1.f, invk = 1.f;
@@ -655,6 +659,20 @@ __global__ __launch_bounds__(NT) void qkv_rows_vec8_kernel(const bf16* __restric
       const float inv = is_q ? invq : invk;
 #pragma unroll
       for (int e = 0; e < 8; ++e) c.v[e] = from_float<bf16>(to_float(c.v[e]) * inv * ws[e]);
+    }
+    if (rot) {                    // the pair (c, c + rot / 2) of a head turns by the position's angle (no norm with it)
+      const int ch = i % d;       // heads and rot / 2 in eights: a piece lies in one half
+      if (ch < rot) {
+        const bool lo = ch < half;
+        const bf16x8_t o = *reinterpret_cast<const bf16x8_t*>(row + (lo ? i + half : i - half));
+        const int a = lo ? ch : ch - half;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float cs = cos_t[trow + a + e], sn = sin_t[trow + a + e];
+          const float x = to_float(c.v[e]), y = to_float(o.v[e]);
+          c.v[e] = from_float<bf16>(lo ? x * cs - y * sn : x * cs + y * sn);
+        }
+      }
     }
     if (is_q) {
       *reinterpret_cast<bf16x8_t*>(q_out + (size_t)t * nqd + i) = c;
@@ -696,9 +714,23 @@ __global__ __launch_bounds__(NT) void qkv_rows_kernel(const T* __restrict__ qkv,
                                                       const T* __restrict__ v_other, long long v_other_stride, float mix,
                                                       const long long* __restrict__ slots, T* __restrict__ q_out,
                                                       T* __restrict__ k_cache, T* __restrict__ v_cache, int page_size,
-                                                      int nq, int nkv, int d, int dv, int v_grouped) {
+                                                      int nq, int nkv, int d, int dv, int v_grouped,
+                                                      const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                      int rot, const int* __restrict__ positions) {
   __shared__ float scratch[NT / kWave];
   const int t = blockIdx.x;
+  const int half = rot / 2;
+  const size_t trow = rot ? (size_t)positions[t] * half : 0;
+  // element i of the q or k part (heads of d) after the rotation of the pair (c, c + rot / 2) by the position's angle
+  auto turned = [&](const T* part, int i, float x) {
+    const int ch = i % d;
+    if (ch >= rot) return x;
+    const bool lo = ch < half;
+    const int a = lo ? ch : ch - half;
+    const float y = to_float(part[lo ? i + half : i - half]);
+    const float cs = cos_t[trow + a], sn = sin_t[trow + a];
+    return lo ? x * cs - y * sn : x * cs + y * sn;
+  };
   const int nqd = nq * d, nkd = nkv * d, nvd = nkv * dv;
   const T* row = qkv + (size_t)t * (nqd + nkd + nvd);
   float invq = 1.f, invk = 1.f;
@@ -717,7 +749,7 @@ __global__ __launch_bounds__(NT) void qkv_rows_kernel(const T* __restrict__ qkv,
     invk = rsqrtf(block_sum<NT / kWave>(ss, scratch) / (float)nkd + eps);
   }
   for (int i = threadIdx.x; i < nqd; i += NT)
-    q_out[(size_t)t * nqd + i] = from_float<T>(qw ? to_float(row[i]) * invq * qw[i] : to_float(row[i]));
+    q_out[(size_t)t * nqd + i] = from_float<T>(qw ? to_float(row[i]) * invq * qw[i] : turned(row, i, to_float(row[i])));
   const long long slot = slots[t];
   if (slot < 0) return;
   const size_t page = (size_t)(slot / page_size);
@@ -725,7 +757,7 @@ __global__ __launch_bounds__(NT) void qkv_rows_kernel(const T* __restrict__ qkv,
   for (int i = threadIdx.x; i < nkd; i += NT) {
     const int h = i / d, c = i - h * d;
     const float v = to_float(row[nqd + i]);
-    k_cache[((page * nkv + h) * page_size + off) * d + c] = from_float<T>(kw ? v * invk * kw[i] : v);
+    k_cache[((page * nkv + h) * page_size + off) * d + c] = from_float<T>(kw ? v * invk * kw[i] : turned(row + nqd, i, v));
   }
   const T* vo = v_other ? v_other + (size_t)t * v_other_stride : nullptr;
   for (int i = threadIdx.x; i < nvd; i += NT) {
@@ -738,7 +770,95 @@ __global__ __launch_bounds__(NT) void qkv_rows_kernel(const T* __restrict__ qkv,
   }
 }
 
+// acc = (acc or 0) + factor * y, float32, y rows or a stack [parts, n] of float32 partial sums added in order
+template <typename T>
+__global__ void scaled_sum_kernel(float* __restrict__ acc, int first, const T* __restrict__ y, int parts, size_t n, float factor) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float s = to_float(y[i]);
+  for (int p = 1; p < parts; ++p) s += to_float(y[(size_t)p * n + i]);
+  acc[i] = first ? factor * s : fmaf(factor, s, acc[i]);
+}
+
+// x *= factor
+__global__ void scale_kernel(float* __restrict__ x, size_t n, float factor) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] *= factor;
+}
+
+// An activation without a gate, in place: 2 = the square of relu (0 and 1 as in act_mul).
+template <typename T, int ACT>
+__global__ void act_kernel(T* __restrict__ x, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float z = to_float(x[i]);
+  float r;
+  if constexpr (ACT == 2) r = z > 0.f ? z * z : 0.f;
+  else r = act_of<ACT>(z);
+  x[i] = from_float<T>(r);
+}
+
+// out[t, :] += sigmoid(gate[t * gate_stride]) * y[t, :]   (out float32; one number a token opens the branch)
+template <typename T>
+__global__ void gated_add_kernel(float* __restrict__ out, const T* __restrict__ y, const float* __restrict__ gate,
+                                 int gate_stride, int H, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const size_t t = i / H;
+  const float g = gate[t * gate_stride];
+  out[i] = fmaf(1.f / (1.f + expf(-g)), to_float(y[i]), out[i]);
+}
+
 extern "C" {
+
+int xi_scaled_sum(float* acc, int first, const void* y, int dtype, int parts, int64_t n, float factor, hipStream_t stream) {
+  XI_CHECK(n >= 0 && parts >= 1, "scaled_sum: bad sizes");
+  if (n == 0) return 0;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (dtype == kF32) scaled_sum_kernel<float><<<blocks, 256, 0, stream>>>(acc, first, (const float*)y, parts, (size_t)n, factor);
+  else if (dtype == kBF16) scaled_sum_kernel<bf16><<<blocks, 256, 0, stream>>>(acc, first, (const bf16*)y, parts, (size_t)n, factor);
+  else XI_CHECK(false, "scaled_sum: unknown dtype %d", dtype);
+  XI_LAUNCH_CHECK("scaled_sum");
+  return 0;
+}
+
+int xi_scale(float* x, int64_t n, float factor, hipStream_t stream) {
+  XI_CHECK(n >= 0, "scale: bad size");
+  if (n == 0) return 0;
+  scale_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, (size_t)n, factor);
+  XI_LAUNCH_CHECK("scale");
+  return 0;
+}
+
+int xi_act(void* x, int dtype, int act, int64_t n, hipStream_t stream) {
+  XI_CHECK(n >= 0 && act >= 0 && act <= 2, "act: bad size or unknown activation %d", act);
+  if (n == 0) return 0;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+#define XI_ACT(TT)                                                                  \
+  do {                                                                              \
+    if (act == 0) act_kernel<TT, 0><<<blocks, 256, 0, stream>>>((TT*)x, (size_t)n); \
+    else if (act == 1) act_kernel<TT, 1><<<blocks, 256, 0, stream>>>((TT*)x, (size_t)n); \
+    else act_kernel<TT, 2><<<blocks, 256, 0, stream>>>((TT*)x, (size_t)n);          \
+  } while (0)
+  if (dtype == kF32) XI_ACT(float);
+  else if (dtype == kBF16) XI_ACT(bf16);
+  else XI_CHECK(false, "act: unknown dtype %d", dtype);
+#undef XI_ACT
+  XI_LAUNCH_CHECK("act");
+  return 0;
+}
+
+int xi_gated_add(float* out, const void* y, int dtype, const float* gate, int gate_stride, int n_tok, int H, hipStream_t stream) {
+  XI_CHECK(n_tok >= 0 && H > 0 && gate_stride > 0, "gated_add: bad sizes T=%d H=%d", n_tok, H);
+  if (n_tok == 0) return 0;
+  const size_t total = (size_t)n_tok * H;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  if (dtype == kF32) gated_add_kernel<float><<<blocks, 256, 0, stream>>>(out, (const float*)y, gate, gate_stride, H, total);
+  else if (dtype == kBF16) gated_add_kernel<bf16><<<blocks, 256, 0, stream>>>(out, (const bf16*)y, gate, gate_stride, H, total);
+  else XI_CHECK(false, "gated_add: unknown dtype %d", dtype);
+  XI_LAUNCH_CHECK("gated_add");
+  return 0;
+}
 
 const char* xi_last_error() { return g_error; }
 
@@ -786,8 +906,9 @@ int xi_softcap(float* x, int64_t n, float cap, hipStream_t stream) {
 
 // y may be null (no add).  rows may be null (all n_rows rows in place).
 // y: null, [T, H], or `parts` partial sums [parts, T, H] (T = resid_rows), added in order.
+// The stream gets resid + y_scale * y (y_scale 1 for the plain sum).
 int xi_add_rmsnorm(float* resid, const void* y, int y_dtype, int parts, int resid_rows, const float* w, float eps,
-                   void* out, int out_dtype, const int* rows, int n_rows, int H, hipStream_t stream) {
+                   void* out, int out_dtype, const int* rows, int n_rows, int H, float y_scale, hipStream_t stream) {
   XI_CHECK(n_rows >= 0 && H > 0, "add_rmsnorm: bad sizes rows=%d H=%d", n_rows, H);
   XI_CHECK(parts >= 1 && resid_rows >= 0, "add_rmsnorm: bad partial sums (%d parts of %d rows)", parts, resid_rows);
   const size_t part_stride = (size_t)resid_rows * H;
@@ -803,14 +924,14 @@ int xi_add_rmsnorm(float* resid, const void* y, int y_dtype, int parts, int resi
   do {                                                                                             \
     if (few)                                                                                       \
       add_rmsnorm_vec_kernel<TY, TO, 1024, 2, 8><<<n_rows, 1024, 0, stream>>>(                     \
-          resid, (const TY*)y, parts, part_stride, w, eps, (TO*)out, rows, H);                     \
+          resid, (const TY*)y, parts, part_stride, w, eps, (TO*)out, rows, H, y_scale);            \
     else if (vec)                                                                                  \
       add_rmsnorm_vec_kernel<TY, TO, NT, MAXV, 4><<<n_rows, NT, 0, stream>>>(                      \
-          resid, (const TY*)y, parts, part_stride, w, eps, (TO*)out, rows, H);                     \
+          resid, (const TY*)y, parts, part_stride, w, eps, (TO*)out, rows, H, y_scale);            \
     else                                                                                           \
       add_rmsnorm_kernel<TY, TO, NT><<<n_rows, NT, 0, stream>>>(resid, (const TY*)y, parts,        \
                                                                 part_stride, w, eps, (TO*)out,     \
-                                                                rows, H);                          \
+                                                                rows, H, y_scale);                 \
   } while (0)
   if (y_dtype == kF32 && out_dtype == kF32) XI_NORM(float, float);
   else if (y_dtype == kBF16 && out_dtype == kBF16) XI_NORM(bf16, bf16);
@@ -975,7 +1096,11 @@ int xi_act_mul(const void* gate_up, void* out, int dtype, int act, int n_tok, in
 // qkv [T, nq d + nkv d + nkv dv]; v_other null or rows of v_other_stride elements holding [nkv dv] values each.
 int xi_qkv_rows(const void* qkv, int dtype, const float* qw, const float* kw, float eps, const void* v_other,
                 long long v_other_stride, float mix, const long long* slots, void* q_out, void* k_cache, void* v_cache,
-                int page_size, int n_tok, int nq, int nkv, int d, int dv, int v_grouped, hipStream_t stream) {
+                int page_size, int n_tok, int nq, int nkv, int d, int dv, int v_grouped, const float* cos_t, const float* sin_t,
+                int rot, const int* positions, hipStream_t stream) {
+  XI_CHECK(rot >= 0 && rot % 2 == 0 && rot <= d, "qkv_rows: %d rotated dims of a head of %d", rot, d);
+  XI_CHECK(rot == 0 || (cos_t && sin_t && positions), "qkv_rows: a rotation needs its tables and the positions");
+  XI_CHECK(rot == 0 || qw == nullptr, "qkv_rows: a rotation and a norm over the whole projection do not go together");
   XI_CHECK(n_tok >= 0 && nq > 0 && nkv > 0 && d > 0 && dv > 0 && page_size > 0,
            "qkv_rows: bad sizes T=%d nq=%d nkv=%d d=%d dv=%d page=%d", n_tok, nq, nkv, d, dv, page_size);
   XI_CHECK((qw == nullptr) == (kw == nullptr), "qkv_rows: q and k norm weights must both be given or both absent");
@@ -984,20 +1109,20 @@ int xi_qkv_rows(const void* qkv, int dtype, const float* qw, const float* kw, fl
   XI_CHECK(v_other == nullptr || v_other_stride >= (long long)nkv * dv, "qkv_rows: the other values' rows are too short");
   if (n_tok == 0) return 0;
   constexpr int NT = 256;
-  if (dtype == kBF16 && d % 8 == 0 && dv % 8 == 0 && (v_other == nullptr || v_other_stride % 8 == 0) &&
+  if (dtype == kBF16 && d % 8 == 0 && dv % 8 == 0 && rot % 16 == 0 && (v_other == nullptr || v_other_stride % 8 == 0) &&
       ((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)v_other | (uintptr_t)qw |
        (uintptr_t)kw) % 16 == 0)
     qkv_rows_vec8_kernel<NT><<<n_tok, NT, 0, stream>>>((const bf16*)qkv, qw, kw, eps, (const bf16*)v_other, v_other_stride, mix,
                                                        slots, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, page_size, nq, nkv,
-                                                       d, dv, v_grouped);
+                                                       d, dv, v_grouped, cos_t, sin_t, rot, positions);
   else if (dtype == kF32)
     qkv_rows_kernel<float, NT><<<n_tok, NT, 0, stream>>>((const float*)qkv, qw, kw, eps, (const float*)v_other, v_other_stride,
                                                          mix, slots, (float*)q_out, (float*)k_cache, (float*)v_cache,
-                                                         page_size, nq, nkv, d, dv, v_grouped);
+                                                         page_size, nq, nkv, d, dv, v_grouped, cos_t, sin_t, rot, positions);
   else if (dtype == kBF16)
     qkv_rows_kernel<bf16, NT><<<n_tok, NT, 0, stream>>>((const bf16*)qkv, qw, kw, eps, (const bf16*)v_other, v_other_stride,
                                                         mix, slots, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, page_size,
-                                                        nq, nkv, d, dv, v_grouped);
+                                                        nq, nkv, d, dv, v_grouped, cos_t, sin_t, rot, positions);
   else
     XI_CHECK(false, "qkv_rows: unknown dtype %d", dtype);
   XI_LAUNCH_CHECK("qkv_rows");

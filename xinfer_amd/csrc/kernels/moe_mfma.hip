@@ -9,7 +9,8 @@
 //                 32 of them; operands come straight from memory, 16 bytes a lane (a row's 64 bytes
 //                 of a K step lie side by side), and stay in registers for MI x 2 products.
 //                 Gated form: W = [gate; up] rows, result act(gate) * up in bfloat16 (the experts'
-//                 hidden rows, kept in slot order); plain form: float32.
+//                 hidden rows, kept in slot order); activated form: W the up rows alone, result
+//                 act(up) in bfloat16 (experts without a gate); plain form: float32.
 //   moe_combine   out[t] = sum over the token's chosen experts, in the order they were chosen, of
 //                 weight * row: a fixed order, float32.
 // A row's result depends on its own operands alone (the matrix cores keep rows apart), so it does not
@@ -63,6 +64,7 @@ __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(const int* __res
 
 template <int ACT>
 __device__ __forceinline__ float moe_act_m(float z) {
+  if constexpr (ACT == 2) return z > 0.f ? z * z : 0.f;       // the square of relu
   if constexpr (ACT == 0) return z / (1.f + __expf(-z));
   else return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
@@ -75,13 +77,15 @@ static __device__ __forceinline__ mbf16x8 mzero8() {
   return z;
 }
 
-// MI: row tiles of 16 a workgroup (its tile has up to 16 * MI rows).  GATED: see the head of the file.
-template <int MI, bool GATED, int ACT>
+// MI: row tiles of 16 a workgroup (its tile has up to 16 * MI rows).  FORM: 0 plain, 1 gated, 2 activated (see
+// the head of the file); the last two read their rows from x through `order`.
+template <int MI, int FORM, int ACT>
 __global__ __launch_bounds__(256) void moe_group_kernel(const bf16* __restrict__ A, const int* __restrict__ order, int top,
                                                         const bf16* __restrict__ W, const int* __restrict__ tile_expert,
                                                         const int* __restrict__ tile_row0, const int* __restrict__ tile_rows,
                                                         const int* __restrict__ n_tiles, void* __restrict__ out, int N,
                                                         int K) {
+  constexpr bool GATED = FORM == 1, GATHER = FORM != 0;
   const int tile = blockIdx.x;
   if (tile >= *n_tiles) return;
   const int e = tile_expert[tile], row0 = tile_row0[tile], rows = tile_rows[tile];
@@ -94,7 +98,7 @@ __global__ __launch_bounds__(256) void moe_group_kernel(const bf16* __restrict__
   for (int i = 0; i < MI; ++i) {
     int slot = row0 + 16 * i + r;
     slot = slot < row0 + rows ? slot : row0 + rows - 1;
-    const size_t arow = GATED ? (size_t)(order[slot] / top) : (size_t)slot;
+    const size_t arow = GATHER ? (size_t)(order[slot] / top) : (size_t)slot;
     ap[i] = A + arow * K;
   }
   constexpr int NB = GATED ? 4 : 2;
@@ -139,6 +143,8 @@ __global__ __launch_bounds__(256) void moe_group_kernel(const bf16* __restrict__
         const size_t at = (size_t)(row0 + row) * N + col;
         if (GATED)
           reinterpret_cast<bf16*>(out)[at] = __float2bfloat16(moe_act_m<ACT>(acc[i][c][v]) * acc[i][GATED ? 2 + c : c][v]);
+        else if (FORM == 2)
+          reinterpret_cast<bf16*>(out)[at] = __float2bfloat16(moe_act_m<ACT>(acc[i][c][v]));
         else
           reinterpret_cast<float*>(out)[at] = acc[i][c][v];
       }
@@ -149,7 +155,7 @@ __global__ __launch_bounds__(256) void moe_group_kernel(const bf16* __restrict__
 // from memory once a workgroup instead of once a wave (two buffers, one barrier a K step; a row of 32 k is padded
 // by 16 bytes against bank conflicts), the weights' operand stays with the wave that owns its features, and every
 // operand of a K step feeds 8 x NB products.  The next step's loads are in flight while this one is multiplied.
-template <bool GATED, int ACT>
+template <int FORM, int ACT>
 __global__ __launch_bounds__(256) void moe_group_lds_kernel(const bf16* __restrict__ A, const int* __restrict__ order, int top,
                                                             const bf16* __restrict__ W, const int* __restrict__ tile_expert,
                                                             const int* __restrict__ tile_row0,
@@ -157,6 +163,7 @@ __global__ __launch_bounds__(256) void moe_group_lds_kernel(const bf16* __restri
                                                             void* __restrict__ out, int N, int K) {
   constexpr int MI = 8, BM = 128, LDA = 32 + 8;
   __shared__ __align__(16) bf16 As[2][BM * LDA];
+  constexpr bool GATED = FORM == 1, GATHER = FORM != 0;
   const int tile = blockIdx.x;
   if (tile >= *n_tiles) return;
   const int e = tile_expert[tile], row0 = tile_row0[tile], rows = tile_rows[tile];
@@ -172,7 +179,7 @@ __global__ __launch_bounds__(256) void moe_group_lds_kernel(const bf16* __restri
     ach[i] = 8 * (idx & 3);
     int slot = row0 + row;
     slot = slot < row0 + rows ? slot : row0 + rows - 1;
-    const size_t arow = GATED ? (size_t)(order[slot] / top) : (size_t)slot;
+    const size_t arow = GATHER ? (size_t)(order[slot] / top) : (size_t)slot;
     agp[i] = A + arow * K + ach[i];
     adst[i] = row * LDA + ach[i];
   }
@@ -240,6 +247,8 @@ __global__ __launch_bounds__(256) void moe_group_lds_kernel(const bf16* __restri
         const size_t at = (size_t)(row0 + row) * N + col;
         if (GATED)
           reinterpret_cast<bf16*>(out)[at] = __float2bfloat16(moe_act_m<ACT>(acc[i][c][v]) * acc[i][GATED ? 2 + c : c][v]);
+        else if (FORM == 2)
+          reinterpret_cast<bf16*>(out)[at] = __float2bfloat16(moe_act_m<ACT>(acc[i][c][v]));
         else
           reinterpret_cast<float*>(out)[at] = acc[i][c][v];
       }
@@ -274,35 +283,43 @@ int xi_moe_sort(const int* idx, int P, int E, int bm, int* order, int* slot_of, 
   return 0;
 }
 
-// gated: A = x [T, K] (row of a slot: order[slot] / top), W [E, 2N, K], out bfloat16 [P, N] = act(gate) * up;
-// plain: A [P, K] in slot order, W [E, N, K], out float32 [P, N].  K a multiple of 8.
+// form 1 (gated): A = x [T, K] (row of a slot: order[slot] / top), W [E, 2N, K], out bfloat16 [P, N] = act(gate) * up;
+// form 2 (activated): the same rows, W [E, N, K], out bfloat16 [P, N] = act(up);
+// form 0 (plain): A [P, K] in slot order, W [E, N, K], out float32 [P, N].  K a multiple of 8.
+// act: 0 silu, 1 gelu (tanh form), 2 the square of relu.
 int xi_moe_group(const void* A, const int* order, int top, const void* W, const int* tile_expert, const int* tile_row0,
-                 const int* tile_rows, const int* n_tiles, int tiles_most, void* out, int N, int K, int bm, int gated, int act,
+                 const int* tile_rows, const int* n_tiles, int tiles_most, void* out, int N, int K, int bm, int form, int act,
                  hipStream_t stream) {
   XI_CHECK(N > 0 && K > 0 && K % 8 == 0 && top > 0 && tiles_most > 0 && (bm == 32 || bm == 64 || bm == 128),
            "moe_group: bad sizes N=%d K=%d (a multiple of 8) top=%d tiles=%d rows=%d", N, K, top, tiles_most, bm);
-  XI_CHECK(act == 0 || act == 1, "moe_group: unknown activation %d", act);
+  XI_CHECK(act >= 0 && act <= 2 && form >= 0 && form <= 2, "moe_group: unknown activation %d or form %d", act, form);
   dim3 grid((unsigned)tiles_most, (unsigned)((N + 127) / 128));
   XI_CHECK(grid.y <= 65535u, "moe_group: N=%d is too large", N);
 #define XI_MG(MI, G, ACT_)                                                                                            \
   moe_group_kernel<MI, G, ACT_><<<grid, 256, 0, stream>>>((const bf16*)A, order, top, (const bf16*)W, tile_expert,    \
                                                           tile_row0, tile_rows, n_tiles, out, N, K)
-  if (bm == 128) {
-    if (!gated) moe_group_lds_kernel<false, 0><<<grid, 256, 0, stream>>>((const bf16*)A, order, top, (const bf16*)W, tile_expert,
-                                                                         tile_row0, tile_rows, n_tiles, out, N, K);
-    else if (act == 0) moe_group_lds_kernel<true, 0><<<grid, 256, 0, stream>>>((const bf16*)A, order, top, (const bf16*)W,
-                                                                               tile_expert, tile_row0, tile_rows, n_tiles, out, N, K);
-    else moe_group_lds_kernel<true, 1><<<grid, 256, 0, stream>>>((const bf16*)A, order, top, (const bf16*)W, tile_expert,
-                                                                 tile_row0, tile_rows, n_tiles, out, N, K);
-  } else if (bm == 32) {
-    if (!gated) XI_MG(2, false, 0);
-    else if (act == 0) XI_MG(2, true, 0);
-    else XI_MG(2, true, 1);
-  } else {
-    if (!gated) XI_MG(4, false, 0);
-    else if (act == 0) XI_MG(4, true, 0);
-    else XI_MG(4, true, 1);
-  }
+#define XI_ML(G, ACT_)                                                                                                \
+  moe_group_lds_kernel<G, ACT_><<<grid, 256, 0, stream>>>((const bf16*)A, order, top, (const bf16*)W, tile_expert,    \
+                                                          tile_row0, tile_rows, n_tiles, out, N, K)
+#define XI_FORMS(LAUNCH, ...)                        \
+  do {                                               \
+    if (form == 0) LAUNCH(__VA_ARGS__ 0, 0);         \
+    else if (form == 1 && act == 0) LAUNCH(__VA_ARGS__ 1, 0); \
+    else if (form == 1 && act == 1) LAUNCH(__VA_ARGS__ 1, 1); \
+    else if (form == 1) LAUNCH(__VA_ARGS__ 1, 2);    \
+    else if (act == 0) LAUNCH(__VA_ARGS__ 2, 0);     \
+    else if (act == 1) LAUNCH(__VA_ARGS__ 2, 1);     \
+    else LAUNCH(__VA_ARGS__ 2, 2);                   \
+  } while (0)
+#define XI_MG2(G, ACT_) XI_MG(2, G, ACT_)
+#define XI_MG4(G, ACT_) XI_MG(4, G, ACT_)
+  if (bm == 128) XI_FORMS(XI_ML);
+  else if (bm == 32) XI_FORMS(XI_MG2);
+  else XI_FORMS(XI_MG4);
+#undef XI_MG2
+#undef XI_MG4
+#undef XI_FORMS
+#undef XI_ML
 #undef XI_MG
   XI_LAUNCH_CHECK("moe_group");
   return 0;

@@ -43,8 +43,20 @@ def load_model(model_dir: str, dtype, device="cuda:0", yarn_scaling_factor: Opti
         store.close()
 
 
+class ShapedNames(list):
+    """The names of a store's tensors, as a list, that can also tell a tensor's shape: for a family that
+    reads a size from its checkpoint where config.json does not name it."""
+
+    def __init__(self, store: WeightStore):
+        super().__init__(store.names())
+        self._store = store
+
+    def shape_of(self, name: str):
+        return tuple(self._store.shape(name))
+
+
 def build_model(config, store: WeightStore, dtype, device="cuda:0") -> CausalLM:
     fam = family_of(config.architecture)
-    model = CausalLM(fam.spec(config, store.names()), parse_dtype(dtype))
+    model = CausalLM(fam.spec(config, ShapedNames(store)), parse_dtype(dtype))
     model.config = config
     return model.load(store, device)

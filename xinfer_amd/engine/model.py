@@ -24,7 +24,7 @@ from ..weights.store import TensorDecl, WeightStore
 class CacheGroupNeed:
     """Layers whose cache needs are the same kind: all keys (window 0) or a window."""
     window: int
-    layers: Tuple[int, ...]             # layer indices that own pages in this group
+    layers: Tuple[int, ...]             # keys of the caches in this group (layer indices, or runs' cache ids)
 
 
 class CausalLM:
@@ -40,7 +40,11 @@ class CausalLM:
         for e in spec.schedule:
             if not (0 <= e.layer < len(self.blocks)):
                 raise ValueError(f"schedule names layer {e.layer} but the model has {len(self.blocks)}")
-            if e.cache_of is not None and not (0 <= e.cache_of < len(self.blocks)):
+            if e.cache_of is not None and e.cache_id is not None:
+                raise ValueError("a schedule entry reads another run's cache or keeps one of its own, not both")
+        ids = {e.cache_id for e in spec.schedule if e.cache_id is not None}
+        for e in spec.schedule:
+            if e.cache_of is not None and e.cache_of not in ids and not (0 <= e.cache_of < len(self.blocks)):
                 raise ValueError(f"schedule entry reads the cache of unknown layer {e.cache_of}")
         self._plan_cache()
 
@@ -81,31 +85,47 @@ class CausalLM:
 
     # ---- cache planning --------------------------------------------------------
     def _plan_cache(self) -> None:
-        """Which layers own pages, in which group; which own per-request state."""
+        """Which runs own pages, in which group; which own per-request state.  A cache is known by a key:
+        the layer's index, or the `cache_id` of a run that keeps one of its own."""
         self.kv_needs: Dict[int, KVNeed] = {}
         self.state_needs: Dict[int, StateNeed] = {}
+        layer_of: Dict[int, int] = {}
+        for e in self.spec.schedule:
+            if e.cache_of is None:
+                key = e.layer if e.cache_id is None else e.cache_id
+                if layer_of.setdefault(key, e.layer) != e.layer:
+                    raise ValueError(f"cache {key} is kept by runs of layers {layer_of[key]} and {e.layer}")
         owners = []
         for e in self.spec.schedule:
-            owner = e.layer if e.cache_of is None else e.cache_of
+            owner = self.cache_key(e)
             if owner not in owners:
                 owners.append(owner)
+                layer_of.setdefault(owner, owner)      # a cache that is only ever read: laid out as that layer's
         windows: List[int] = []
         by_window: Dict[int, List[int]] = {}
-        for l in owners:
+        for key in owners:
+            l = layer_of[key]
             kv = self.blocks[l].cache_need()
             if kv is not None:
-                self.kv_needs[l] = kv
+                self.kv_needs[key] = kv
                 if kv.window not in by_window:
                     by_window[kv.window] = []
                     windows.append(kv.window)
-                by_window[kv.window].append(l)
+                by_window[kv.window].append(key)
             st = self.blocks[l].state_need()
             if st is not None:
-                self.state_needs[l] = st
+                self.state_needs[key] = st
         self.cache_groups: List[CacheGroupNeed] = [
             CacheGroupNeed(w, tuple(by_window[w])) for w in windows]
         self.group_of_layer: Dict[int, int] = {
             l: g for g, grp in enumerate(self.cache_groups) for l in grp.layers}
+
+    @staticmethod
+    def cache_key(e) -> int:
+        """The key of the cache that a schedule entry's run uses."""
+        if e.cache_of is not None:
+            return e.cache_of
+        return e.layer if e.cache_id is None else e.cache_id
 
     # ---- step ------------------------------------------------------------------
     def forward(self, ids: torch.Tensor, ctx: StepContext, caches: Dict[int, LayerCache],
@@ -117,8 +137,7 @@ class CausalLM:
         stream = Stream(first, None, rows=getattr(self.embedding, "rows", None))
         schedule = self.spec.schedule
         for i, e in enumerate(schedule):
-            owner = e.layer if e.cache_of is None else e.cache_of
-            c = caches.get(owner)
+            c = caches.get(self.cache_key(e))
             if c is None:
                 c = LayerCache()
             elif e.cache_of is not None:
@@ -131,5 +150,9 @@ class CausalLM:
                 stream = blk.forward(stream, ctx, c, next_norm=next_norm)
             else:
                 stream = blk.forward(stream, ctx, c)
-        h = self.final_norm.forward(stream.resid, stream.pending, self.dtype, rows=want_rows)
+        if stream.pending is not None and stream.pending_scale != 1.0:
+            h = self.final_norm.forward(stream.resid, stream.pending, self.dtype, rows=want_rows,
+                                        add_scale=stream.pending_scale)
+        else:
+            h = self.final_norm.forward(stream.resid, stream.pending, self.dtype, rows=want_rows)
         return self.head.forward(h)

@@ -31,7 +31,7 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at a time, each rounded up to a page")
     ap.add_argument("--page-size", type=int, default=64, help="tokens per cache page")
-    ap.add_argument("--max-requests", type=int, default=8, help="most live requests at a time")
+    ap.add_argument("--max-requests", type=int, default=4, help="most live requests at a time (state slots)")
     args = ap.parse_args(argv)
 
     print("trace_run: loading (kernels are compiled on the first call)", file=sys.stderr, flush=True)

@@ -144,8 +144,8 @@ def softcap_(logits: torch.Tensor, cap: float) -> torch.Tensor:
 
 def add_rmsnorm(resid: torch.Tensor, y: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
-                out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """s = resid (+ y); out = rms(s) * weight in `out_dtype`.  Without `rows` every row is
+                out: Optional[torch.Tensor] = None, y_scale: float = 1.0) -> torch.Tensor:
+    """s = resid (+ y_scale * y); out = rms(s) * weight in `out_dtype`.  Without `rows` every row is
     normed and the sum is written back into resid; with `rows` (int32 indices) only those
     rows are produced and resid is left alone.  y may be a stack [P, T, H] of float32 partial
     sums, which are added in order."""
@@ -173,7 +173,7 @@ def add_rmsnorm(resid: torch.Tensor, y: Optional[torch.Tensor], weight: torch.Te
         raise KernelError("add_rmsnorm: out has the wrong shape or dtype")
     _ok(lib().xi_add_rmsnorm(_p(resid), _p(y), _code(y, "add_rmsnorm") if y is not None else F32, parts,
                              int(resid.shape[0]), _p(weight), ctypes.c_float(eps), _p(out),
-                             _code(out, "add_rmsnorm"), _p(rows), n, H, _stream()))
+                             _code(out, "add_rmsnorm"), _p(rows), n, H, ctypes.c_float(y_scale), _stream()))
     return out
 
 
@@ -192,6 +192,133 @@ def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
 
 
 ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+UNGATED_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "relu2": 2}     # relu2: the square of relu
+
+
+def act_(x: torch.Tensor, act: str) -> torch.Tensor:
+    """x <- act(x) in place, an activation without a gate (see UNGATED_ACTIVATIONS)."""
+    _dev(x)
+    if act not in UNGATED_ACTIVATIONS:
+        raise KernelError(f"act: unknown activation {act!r}")
+    _ok(lib().xi_act(_p(x), _code(x, "act"), UNGATED_ACTIVATIONS[act], ctypes.c_int64(x.numel()), _stream()))
+    return x
+
+
+def scaled_sum(acc: Optional[torch.Tensor], y: torch.Tensor, factor: float) -> torch.Tensor:
+    """acc + factor * y in float32 (acc None: factor * y in a new tensor; else in place).  y: rows [T, H] in
+    either precision, or a stack [P, T, H] of float32 partial sums, which are added in order first."""
+    _dev(acc, y)
+    parts = 1
+    if y.dim() == 3:
+        _want(y, torch.float32, "scaled_sum: partial sums")
+        parts = int(y.shape[0])
+    elif y.dim() != 2:
+        raise KernelError("scaled_sum: rows [T, H] or partial sums [P, T, H]")
+    shape = tuple(y.shape[-2:])
+    first = acc is None
+    if first:
+        acc = torch.empty(shape, dtype=torch.float32, device=y.device)
+    elif acc.dtype != torch.float32 or tuple(acc.shape) != shape:
+        raise KernelError(f"scaled_sum: the sum {tuple(acc.shape)} {acc.dtype} must be float32 {shape}")
+    _ok(lib().xi_scaled_sum(_p(acc), int(first), _p(y), _code(y, "scaled_sum"), parts, ctypes.c_int64(acc.numel()),
+                            ctypes.c_float(factor), _stream()))
+    return acc
+
+
+def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:
+    """x <- x * factor in place (float32)."""
+    _dev(x)
+    _want(x, torch.float32, "scale")
+    _ok(lib().xi_scale(_p(x), ctypes.c_int64(x.numel()), ctypes.c_float(factor), _stream()))
+    return x
+
+
+def gated_add_(out: torch.Tensor, y: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """out[t] += sigmoid(gate[t]) * y[t]: out float32 [T, H], y [T, H], gate float32 [T] or a column [T, X][:, 0]
+    (one number a token)."""
+    _dev(out, y)
+    _want(out, torch.float32, "gated_add: out")
+    _want(gate, torch.float32, "gated_add: gate")
+    if out.dim() != 2 or y.shape != out.shape or gate.dim() != 1 or gate.shape[0] != out.shape[0] or not gate.is_cuda:
+        raise KernelError(f"gated_add: out {tuple(out.shape)}, y {tuple(y.shape)} and gate {tuple(gate.shape)} do not match")
+    _ok(lib().xi_gated_add(_p(out), _p(y), _code(y, "gated_add"), _p(gate), int(gate.stride(0)) if gate.shape[0] > 1 else 1,
+                           int(out.shape[0]), int(out.shape[1]), _stream()))
+    return out
+
+
+def _columns(t: torch.Tensor, width: int, what: str):
+    """A [T, width] view of a packed projection: its pointer stays, the row stride is handed to the kernel."""
+    if t.dim() != 2 or t.shape[1] != width or t.stride(1) != 1 or not t.is_cuda:
+        raise KernelError(f"{what}: {tuple(t.shape)} with strides {t.stride()} is not [T, {width}] rows")
+    return int(t.stride(0)) if t.shape[0] > 1 else width
+
+
+def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.Tensor, state_slots: torch.Tensor,
+                cu_q: torch.Tensor, heads: int, key_dim: int, value_dim: int, z: Optional[torch.Tensor] = None,
+                tau: float = 1.0, head_decay: Optional[torch.Tensor] = None, q_scale: float = 1.0,
+                k_scale: float = 1.0, z_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Linear attention with a decaying float32 state per request and head, S <- diag(a) S + k v^T, o = S^T q,
+    token by token from the state each request's slot holds (left there afterwards).  q, k [T, H dk] and
+    v [T, H dv] may be column ranges of a packed projection.  The decay: `z` float32 [T, H dk], `z_bias`
+    float32 [H dk] (or None) and `tau` (a = sigmoid(z + bias)^(1 / tau) per token and key channel) or `head_decay` float32 [H] (a constant per head).
+    state float32 [slots, H, dk, dv] (slots may be strided); state_slots int64 [B]; cu_q int32 [B + 1].
+    Returns o float32 [T, H, dv]."""
+    H, dk, dv = int(heads), int(key_dim), int(value_dim)
+    T = q.shape[0]
+    qs, ks, vs = _columns(q, H * dk, "linear_scan: q"), _columns(k, H * dk, "linear_scan: k"), _columns(v, H * dv, "linear_scan: v")
+    if k.shape[0] != T or v.shape[0] != T or q.dtype != k.dtype or q.dtype != v.dtype or not (q.device == k.device == v.device):
+        raise KernelError("linear_scan: q, k and v must be rows of the same tokens, type and device")
+    _dev(z, head_decay, state_slots, cu_q, z_bias)
+    if z_bias is not None and (z is None or z_bias.dtype != torch.float32 or z_bias.shape != (H * dk,)):
+        raise KernelError(f"linear_scan: the bias of the decay's logits must be float32 [{H * dk}], beside z")
+    if (z is None) == (head_decay is None):
+        raise KernelError("linear_scan: a decay per token (z) or per head (head_decay), one of them")
+    if z is not None:
+        _want(z, torch.float32, "linear_scan: z")
+        if z.shape != (T, H * dk) or not tau > 0:
+            raise KernelError(f"linear_scan: z {tuple(z.shape)} must be [{T}, {H * dk}] and tau positive")
+    else:
+        _want(head_decay, torch.float32, "linear_scan: head_decay")
+        if head_decay.shape != (H,):
+            raise KernelError(f"linear_scan: head_decay {tuple(head_decay.shape)} must be [{H}]")
+    _want(state, torch.float32, "linear_scan: state")
+    _want(state_slots, torch.int64, "linear_scan: state_slots")
+    _want(cu_q, torch.int32, "linear_scan: cu_q")
+    if (state.dim() != 4 or tuple(state.shape[1:]) != (H, dk, dv) or not state.is_cuda or state.device != q.device
+            or state[0].stride() != (dk * dv, dv, 1)):
+        raise KernelError(f"linear_scan: state {tuple(state.shape)} must be [slots, {H}, {dk}, {dv}] with whole slots")
+    B = state_slots.shape[0]
+    if cu_q.shape != (B + 1,) or dk > 256:
+        raise KernelError("linear_scan: cu_q must be [B + 1]; key heads of up to 256 channels")
+    out = torch.empty((T, H, dv), dtype=torch.float32, device=q.device)
+    _ok(lib().xi_linear_scan(_p(q), ctypes.c_longlong(qs), _p(k), ctypes.c_longlong(ks), _p(v), ctypes.c_longlong(vs),
+                             _code(q, "linear_scan"), _p(z), _p(z_bias), ctypes.c_float(tau), _p(head_decay), _p(state),
+                             ctypes.c_longlong(int(state.stride(0)) if state.shape[0] > 1 else H * dk * dv), _p(state_slots),
+                             _p(cu_q), _p(out), B, H, dk, dv, ctypes.c_float(q_scale), ctypes.c_float(k_scale), _stream()))
+    return out
+
+
+def head_norm_gate(o: torch.Tensor, weight: Optional[torch.Tensor], eps: float, gate: torch.Tensor,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """o float32 [T, H, dv]: each head divided by its root mean square over dv (eps inside the root), times
+    `weight` float32 [dv] (shared by the heads; None: no weight), times silu(gate) (gate [T, H dv], may be a
+    column range of a packed projection, in `out_dtype`).  Returns [T, H dv] in `out_dtype`."""
+    _dev(o, weight)
+    _want(o, torch.float32, "head_norm_gate: o")
+    if o.dim() != 3:
+        raise KernelError("head_norm_gate: o must be [T, H, dv]")
+    T, H, dv = o.shape
+    gs = _columns(gate, H * dv, "head_norm_gate: gate")
+    if gate.shape[0] != T or gate.dtype != out_dtype or gate.device != o.device:
+        raise KernelError("head_norm_gate: the gate must be rows of the same tokens in the output's type")
+    if weight is not None:
+        _want(weight, torch.float32, "head_norm_gate: weight")
+        if weight.shape != (dv,):
+            raise KernelError(f"head_norm_gate: weight {tuple(weight.shape)} must be [{dv}]")
+    out = torch.empty((T, H * dv), dtype=out_dtype, device=o.device)
+    _ok(lib().xi_head_norm_gate(_p(o), _p(weight), ctypes.c_float(eps), _p(gate), ctypes.c_longlong(gs), _p(out),
+                                _code(out, "head_norm_gate"), T, H, dv, _stream()))
+    return out
 
 
 def act_mul(gate_up: torch.Tensor, act: str = "silu") -> torch.Tensor:
@@ -257,12 +384,26 @@ def rmsnorm_add(resid: torch.Tensor, y: torch.Tensor, weight: Optional[torch.Ten
 def qkv_rows(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
              slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, num_heads: int, num_kv_heads: int,
              head_dim: int, value_dim: int, v_grouped: bool = False, v_other: Optional[torch.Tensor] = None,
-             mix: float = 0.0) -> torch.Tensor:
+             mix: float = 0.0, cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, rotary_dim: int = 0,
+             positions: Optional[torch.Tensor] = None) -> torch.Tensor:
     """A packed projection [T, nq d + nkv d + nkv dv] made ready for attention without rotation: RMSNorm
     over the whole q part and the whole k part (weights float32 [nq d] and [nkv d]; none: no norm), v
     blended with `v_other` ([T, nkv dv], rows may be a strided view: another layer's values of the same
-    tokens) as (1 - mix) v + mix v_other, k and v into the paged cache at `slots`.  Returns q [T, nq, d]."""
-    _dev(qkv, q_weight, k_weight, slots, k_cache, v_cache)
+    tokens) as (1 - mix) v + mix v_other, k and v into the paged cache at `slots`.  Returns q [T, nq, d].
+    With `rotary_dim` r > 0 (and no norm) the pairs (c, c + r / 2) of every q and k head turn by the token's
+    angles first: `cos` / `sin` float32 [positions, r / 2], `positions` int32 [T]."""
+    _dev(qkv, q_weight, k_weight, slots, k_cache, v_cache, cos, sin, positions)
+    rot = int(rotary_dim)
+    if rot:
+        if q_weight is not None or rot % 2 or not (0 < rot <= int(head_dim)):
+            raise KernelError(f"qkv_rows: {rot} rotated dims of a head of {head_dim} (even, and no norm over the projection)")
+        if cos is None or sin is None or positions is None or cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != rot // 2:
+            raise KernelError(f"qkv_rows: the rotation's tables must be [positions, {rot // 2}]")
+        _want(cos, torch.float32, "qkv_rows: cos")
+        _want(sin, torch.float32, "qkv_rows: sin")
+        _want(positions, torch.int32, "qkv_rows: positions")
+        if positions.shape != (qkv.shape[0],):
+            raise KernelError("qkv_rows: positions must be [T]")
     nq, nkv, d, dv = int(num_heads), int(num_kv_heads), int(head_dim), int(value_dim)
     if qkv.dim() != 2 or qkv.shape[1] != nq * d + nkv * d + nkv * dv:
         raise KernelError(f"qkv_rows: qkv {tuple(qkv.shape)} is not [T, {nq * d + nkv * d + nkv * dv}]")
@@ -286,20 +427,28 @@ def qkv_rows(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Opti
     q_out = torch.empty((T, nq, d), dtype=qkv.dtype, device=qkv.device)
     _ok(lib().xi_qkv_rows(_p(qkv), _code(qkv, "qkv_rows"), _p(q_weight), _p(k_weight), ctypes.c_float(eps), _p(v_other),
                           ctypes.c_longlong(stride), ctypes.c_float(mix), _p(slots), _p(q_out), _p(k_cache), _p(v_cache),
-                          int(k_cache.shape[2]), T, nq, nkv, d, dv, int(bool(v_grouped)), _stream()))
+                          int(k_cache.shape[2]), T, nq, nkv, d, dv, int(bool(v_grouped)), _p(cos if rot else None),
+                          _p(sin if rot else None), rot, _p(positions if rot else None), _stream()))
     return q_out
 
 
-def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int):
+def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int, all_scores: bool = False,
+              extra_rows: int = 0):
     """Router of a mixture of experts: z = router @ x + bias in float32 (router float32 [E, H]), the `top`
-    largest (ties: the lower index), weights = softmax over the chosen logits.  Returns
-    (idx int32 [T, top], weights float32 [T, top]), the chosen in descending order of their logits."""
+    largest (ties: the lower index), weights = softmax over the chosen logits, or with `all_scores` the
+    softmax over all experts, the chosen scores divided by their sum + 1e-20.  Returns
+    (idx int32 [T, top], weights float32 [T, top]), the chosen in descending order of their logits.
+    `extra_rows` X > 0: the router's last X rows are no experts but further float32 products of the same
+    rows (a shared branch's gate); their results come back as a third value, float32 [T, X]."""
     _dev(x, router, bias)
+    X = int(extra_rows)
+    if X < 0 or X >= router.shape[0]:
+        raise KernelError(f"moe_route: {X} further rows of a router of {router.shape[0]}")
     _want(router, torch.float32, "moe_route: router weight")
     if x.dim() != 2 or router.dim() != 2 or router.shape[1] != x.shape[1]:
         raise KernelError(f"moe_route: x {tuple(x.shape)} and the router {tuple(router.shape)} do not match")
     T, H = x.shape
-    E = router.shape[0]
+    E = router.shape[0] - X
     if bias is not None:
         _want(bias, torch.float32, "moe_route: bias")
         if bias.shape != (E,):
@@ -308,8 +457,10 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor
         raise KernelError(f"moe_route: {top} of {E} experts (at most 64 of 1024)")
     idx = torch.empty((T, top), dtype=torch.int32, device=x.device)
     wt = torch.empty((T, top), dtype=torch.float32, device=x.device)
-    _ok(lib().xi_moe_route(_p(x), _code(x, "moe_route"), _p(router), _p(bias), _p(idx), _p(wt), T, H, E, int(top), _stream()))
-    return idx, wt
+    extra = torch.empty((T, X), dtype=torch.float32, device=x.device) if X else None
+    _ok(lib().xi_moe_route(_p(x), _code(x, "moe_route"), _p(router), _p(bias), _p(idx), _p(wt), T, H, E, int(top),
+                           int(bool(all_scores)), _p(extra), X, _stream()))
+    return (idx, wt, extra) if X else (idx, wt)
 
 
 MOE_GROUPED = True        # False: every step takes the experts one (token, expert) pair at a time
@@ -328,7 +479,7 @@ MOE_LIBRARY_ROWS = 64     # rows an expert on average from which a step of porti
 
 
 def moe_experts_library(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx: torch.Tensor, wt: torch.Tensor,
-                        act: str = "silu") -> torch.Tensor:
+                        act: str = "silu", gated: bool = True) -> torch.Tensor:
     """`moe_experts` for steps of many tokens in bfloat16: the pairs sorted by expert on the device, the rows
     gathered in that order, and one plain product of the vendor library an expert and projection (as the
     dense feed-forward's products of many rows go to the library); the hand-written kernels do the sort,
@@ -337,11 +488,13 @@ def moe_experts_library(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tens
     _dev(x, gate_up, down, idx, wt)
     T, H = x.shape
     E, F2, _ = gate_up.shape
-    F, top = F2 // 2, int(idx.shape[1])
+    F, top = (F2 // 2 if gated else F2), int(idx.shape[1])
     if x.dtype != torch.bfloat16 or gate_up.dtype != torch.bfloat16 or down.dtype != torch.bfloat16:
         raise KernelError("moe_experts_library: operands must be bfloat16")
-    if gate_up.shape != (E, 2 * F, H) or down.shape != (E, H, F) or idx.shape != (T, top) or wt.shape != (T, top):
-        raise KernelError("moe_experts_library: x [T, H], gate_up [E, 2F, H], down [E, H, F], idx and weights [T, top]")
+    if act not in (ACTIVATIONS if gated else UNGATED_ACTIVATIONS):
+        raise KernelError(f"moe_experts_library: unknown activation {act!r}")
+    if gate_up.shape != (E, (2 if gated else 1) * F, H) or down.shape != (E, H, F) or idx.shape != (T, top) or wt.shape != (T, top):
+        raise KernelError("moe_experts_library: x [T, H], gate_up [E, 2F, H] (up alone: [E, F, H]), down [E, H, F], idx and weights [T, top]")
     _want(idx, torch.int32, "moe_experts_library: idx")
     _want(wt, torch.float32, "moe_experts_library: weights")
     P = T * top
@@ -357,7 +510,8 @@ def moe_experts_library(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tens
     at = 0
     for e, n in enumerate(counts[:E]):
         if n:
-            mid = act_mul(torch.nn.functional.linear(rows[at:at + n], gate_up[e]), act)
+            mid = torch.nn.functional.linear(rows[at:at + n], gate_up[e])
+            mid = act_mul(mid, act) if gated else act_(mid, act)
             torch.mm(mid, down[e].t(), out_dtype=torch.float32, out=y[at:at + n])
             at += n
     out = torch.empty((T, H), dtype=torch.float32, device=x.device)
@@ -366,21 +520,24 @@ def moe_experts_library(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tens
 
 
 def moe_experts(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx: torch.Tensor, wt: torch.Tensor,
-                act: str = "silu", grouped: Optional[bool] = None, tile_rows: Optional[int] = None) -> torch.Tensor:
+                act: str = "silu", grouped: Optional[bool] = None, tile_rows: Optional[int] = None,
+                gated: bool = True) -> torch.Tensor:
     """sum over a token's chosen experts e (in the order of `idx`) of wt * down[e] @ (act(gate[e] @ x) * (up[e] @ x)):
     gate_up [E, 2F, H] (gate rows first), down [E, H, F], idx int32 / wt float32 [T, top].  Float32 [T, H].
+    `gated` False: experts without a gate, wt * down[e] @ act(up[e] @ x), `gate_up` the up rows alone [E, F, H].
     One (token, expert) pair at a time, every sum in an order fixed by the sizes: the form of the
     float32 path and of steps with few tokens.  `grouped` (None: chosen by `moe_grouped_takes`): the pairs
     sorted by expert on the device and each expert's rows multiplied in tiles on the matrix cores."""
     _dev(x, gate_up, down, idx, wt)
-    if act not in ACTIVATIONS:
+    acts = ACTIVATIONS if gated else UNGATED_ACTIVATIONS
+    if act not in acts:
         raise KernelError(f"moe_experts: unknown activation {act!r}")
     if gate_up.dim() != 3 or down.dim() != 3 or x.dim() != 2:
         raise KernelError("moe_experts: x [T, H], gate_up [E, 2F, H], down [E, H, F]")
     T, H = x.shape
     E, F2, _ = gate_up.shape
-    F = F2 // 2
-    if gate_up.shape != (E, 2 * F, H) or down.shape != (E, H, F) or x.dtype != gate_up.dtype or x.dtype != down.dtype:
+    F = F2 // 2 if gated else F2
+    if gate_up.shape != (E, (2 if gated else 1) * F, H) or down.shape != (E, H, F) or x.dtype != gate_up.dtype or x.dtype != down.dtype:
         raise KernelError(f"moe_experts: x {tuple(x.shape)} {x.dtype}, gate_up {tuple(gate_up.shape)} {gate_up.dtype} and "
                           f"down {tuple(down.shape)} {down.dtype} do not match")
     _want(idx, torch.int32, "moe_experts: idx")
@@ -408,7 +565,7 @@ def moe_experts(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx:
         _ok(lib().xi_moe_sort(_p(idx), P, E, bm, _p(order), _p(slot_of), _p(t_e), _p(t_r0), _p(t_n), _p(n_tiles), _stream()))
         mid = torch.empty((P, F), dtype=torch.bfloat16, device=x.device)
         _ok(lib().xi_moe_group(_p(x), _p(order), top, _p(gate_up), _p(t_e), _p(t_r0), _p(t_n), _p(n_tiles), most, _p(mid),
-                               F, H, bm, 1, ACTIVATIONS[act], _stream()))
+                               F, H, bm, 1 if gated else 2, acts[act], _stream()))
         y = torch.empty((P, H), dtype=torch.float32, device=x.device)
         _ok(lib().xi_moe_group(_p(mid), _p(order), top, _p(down), _p(t_e), _p(t_r0), _p(t_n), _p(n_tiles), most, _p(y),
                                H, F, bm, 0, 0, _stream()))
@@ -416,7 +573,7 @@ def moe_experts(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx:
         return out
     mid = torch.empty((T * top, F), dtype=x.dtype, device=x.device)
     code = _code(x, "moe_experts")
-    _ok(lib().xi_moe_gate_up(_p(x), _p(gate_up), _p(idx), _p(mid), code, ACTIVATIONS[act], T, H, F, E, top, _stream()))
+    _ok(lib().xi_moe_gate_up(_p(x), _p(gate_up), _p(idx), _p(mid), code, acts[act], int(bool(gated)), T, H, F, E, top, _stream()))
     _ok(lib().xi_moe_down(_p(mid), _p(down), _p(idx), _p(wt), _p(out), code, T, H, F, E, top, _stream()))
     return out
 

@@ -15,7 +15,9 @@ and key j; values blended with those another layer made for the same token, (1 -
 (`value_mix`: the layers of one `key` share the values of the one that is their `source`, m is a
 scalar tensor of the layer); other tensor names (`names`).  Any of these takes the step through
 `_forward_general`: one kernel norms the projection, blends the values and writes the cache, and
-the attention kernels that know the score's options follow.
+the attention kernels that know the score's options follow.  That kernel also rotates q and k by
+position (pairs (i, i + rotary_dim / 2), float32 tables) where the spec names a position encoding and
+no q/k norm.
 """
 from __future__ import annotations
 
@@ -62,9 +64,9 @@ class PagedAttention(Mixer):
         # the options that the fused q/k kernel and the attention kernels of the plain form do not know
         self.general = bool(self.dv != self.d or self.row_norm or self.softcap > 0 or self.slope_values is not None
                             or self.value_mix_key is not None)
-        if self.general and spec.get("position") is not None:
-            raise NotImplementedError("attention with a soft cap, a distance bias, a row norm, blended values or another "
-                                      "value size takes no rotation (position encoding) yet")
+        if self.general and spec.get("position") is not None and (self.qk_norm or bool(spec["position"].get("interleaved", False))):
+            raise NotImplementedError("attention with a soft cap, a distance bias, blended values or another value size takes a "
+                                      "rotation of the pairs (i, i + rotary_dim / 2) and then no q/k norm")
         if self.general and (self.qk_norm and not self.row_norm or self.bias):
             raise NotImplementedError("attention with a soft cap, a distance bias, blended values or another value size "
                                       "takes the q/k norm over the whole projection or none, and no biases")
@@ -198,8 +200,11 @@ class PagedAttention(Mixer):
                 v_other = ctx.scratch.get(key)
                 if v_other is None:
                     raise RuntimeError(f"values {self.value_mix_key!r} are blended in before the layer that makes them has run")
+        pos = self.position
         q = kernels.qkv_rows(qkv, self.q_norm_w, self.k_norm_w, self.qk_norm_eps, slots, cache.k, cache.v,
-                             self.nq, self.nkv, self.d, self.dv, v_grouped=vt, v_other=v_other, mix=self.mix)
+                             self.nq, self.nkv, self.d, self.dv, v_grouped=vt, v_other=v_other, mix=self.mix,
+                             cos=pos.cos if pos is not None else None, sin=pos.sin if pos is not None else None,
+                             rotary_dim=pos.rotary_dim if pos is not None else 0, positions=ctx.positions)
         a = kernels.attention(q, cache.k, cache.v, ctx, cache.group, self.scale, self.window, v_grouped=vt,
                               softcap=self.softcap, slopes=self.slopes)
         return self.o(a, out_dtype=self.dtype, allow_split=True, sink=sink)

@@ -13,7 +13,8 @@ runs on the tokens of one step.  A part never learns which model it is in.
   Norm             forward(resid, add, out_dtype, rows=None, out=None) -> normed
                    resid is the float32 residual stream; `add` (if given) is summed into
                    it first; with `rows` only those rows are produced and resid is not
-                   changed.
+                   changed.  A kind that can add `add_scale * add` takes that keyword too
+                   (it is only passed where the factor is not 1).
                    forward_branch(resid, y, rows_dtype): resid += norm(y), for blocks that norm
                    a sublayer's output instead of its input.
   PositionEncoding data for the mixer's fused kernel (for "rope": cos/sin tables)
@@ -170,6 +171,7 @@ class Stream:
     folded: Optional[Folded] = None
     rows: Optional[torch.Tensor] = None       # `resid` rounded to the activation dtype, as it is now (nothing
                                               # pending): what a sublayer that reads the stream itself takes
+    pending_scale: float = 1.0                # the stream is to get pending_scale * pending
 
 
 class Part:

@@ -4,7 +4,9 @@
 (reference: Qwen3DecoderLayer::forward, /root/reference/src/models/qwen3.rs:108-134).
 Each residual add is carried out by the norm kernel that follows it: a block hands on
 the stream with its feed-forward output still pending, and the next block's first
-norm (or the model's final norm) adds it.
+norm (or the model's final norm) adds it.  With the block parameter `residual_scale` m the
+stream gets m times each branch, x <- x + m * mixer(norm(x)), then x <- x + m * ff(norm(x)); a layer
+without a feed-forward ends after the first of the two.
 
 "branchnorm": x <- x + norm1(mixer(x)); x <- x + norm2(ff(x)): the sublayers read the stream
 itself and their OUTPUT is normed; a layer may have no feed-forward.  The norm, the add and
@@ -30,30 +32,40 @@ class PreNormBlock(Block):
     def __init__(self, layer: LayerSpec, dtype: torch.dtype):
         super().__init__(layer, dtype)
         self.mixer = mixer_class(layer.mixer.kind)(layer.mixer, dtype)
-        self.ffn = feed_forward_class(layer.feed_forward.kind)(layer.feed_forward, dtype)
-        (self._name1, n1), (self._name2, n2) = layer.norm_items(2)
+        self.ffn = (feed_forward_class(layer.feed_forward.kind)(layer.feed_forward, dtype)
+                    if layer.feed_forward is not None else None)
+        self.scale = float(layer.block_params.get("residual_scale", 1.0))
+        items = layer.norm_items(2 if self.ffn is not None else 1)
+        self._name1, n1 = items[0]
         self.norm1 = norm_class(n1.kind)(n1, dtype)
-        self.norm2 = norm_class(n2.kind)(n2, dtype)
+        self._name2, self.norm2 = None, None
+        if self.ffn is not None:
+            self._name2, n2 = items[1]
+            self.norm2 = norm_class(n2.kind)(n2, dtype)
+        # a norm rides on the products around it only where the stream gets the plain sum
+        self.folds = self.scale == 1.0 and self.ffn is not None
 
     @classmethod
     def declare(cls, layer: LayerSpec) -> List[TensorDecl]:
         p = layer.prefix
         out = mixer_class(layer.mixer.kind).declare(layer.mixer, f"{p}.{layer.mixer_name}")
-        out += feed_forward_class(layer.feed_forward.kind).declare(layer.feed_forward, f"{p}.{layer.feed_forward_name}")
-        for name, n in layer.norm_items(2):
+        if layer.feed_forward is not None:
+            out += feed_forward_class(layer.feed_forward.kind).declare(layer.feed_forward, f"{p}.{layer.feed_forward_name}")
+        for name, n in layer.norm_items(2 if layer.feed_forward is not None else 1):
             out += norm_class(n.kind).declare(n, f"{p}.{name}")
         return out
 
     def load(self, store: WeightStore, device) -> None:
         p = self.layer.prefix
         self.mixer.load(store, f"{p}.{self.layer.mixer_name}", device)
-        self.ffn.load(store, f"{p}.{self.layer.feed_forward_name}", device)
         self.norm1.load(store, f"{p}.{self._name1}", device)
-        self.norm2.load(store, f"{p}.{self._name2}", device)
+        if self.ffn is not None:
+            self.ffn.load(store, f"{p}.{self.layer.feed_forward_name}", device)
+            self.norm2.load(store, f"{p}.{self._name2}", device)
 
     @property
     def graph_safe(self) -> bool:
-        return all(p.graph_safe for p in (self.mixer, self.ffn, self.norm1, self.norm2))
+        return all(p.graph_safe for p in (self.mixer, self.ffn, self.norm1, self.norm2) if p is not None)
 
     def cache_need(self) -> Optional[KVNeed]:
         return self.mixer.cache_need()
@@ -62,7 +74,7 @@ class PreNormBlock(Block):
         return self.mixer.state_need()
 
     # ---- folding norms into the products around them (parts.base.Folded) ---------------------
-    folds = True         # `forward` takes `next_norm` and a stream with `folded`
+    # `folds` (set per block): `forward` takes `next_norm` and a stream with `folded`
 
     def first_norm(self):
         """The norm that a block before this one may half do, or None."""
@@ -71,10 +83,14 @@ class PreNormBlock(Block):
     def forward(self, stream: Stream, ctx: StepContext, cache: LayerCache, next_norm=None) -> Stream:
         """`next_norm`: the first norm of the block that runs next, if that block lets this
         one's feed-forward half do it."""
+        if not self.folds:
+            return self._forward_scaled(stream, ctx, cache)
         if stream.folded is not None:
             if stream.folded.norm is not self.norm1:
                 raise RuntimeError("the stream carries a half-done norm of another block")
             h = stream.folded
+        elif stream.pending_scale != 1.0:
+            h = self.norm1.forward(stream.resid, stream.pending, self.dtype, add_scale=stream.pending_scale)
         else:
             h = self.norm1.forward(stream.resid, stream.pending, self.dtype)
         if self.mixer.takes_sink and self.ffn.takes_folded and self.norm2.foldable:
@@ -89,6 +105,24 @@ class PreNormBlock(Block):
         if isinstance(m, Folded):
             return Stream(stream.resid, None, m)
         return Stream(stream.resid, m)
+
+    def _forward_scaled(self, stream: Stream, ctx: StepContext, cache: LayerCache) -> Stream:
+        """The step with a factor on the branches, or without a feed-forward: every add is done by the norm
+        kernel that follows it, with its factor."""
+        if stream.folded is not None:
+            raise RuntimeError("the stream carries a half-done norm of another block")
+        resid = stream.resid
+
+        def normed(norm, add, scale):
+            if add is not None and scale != 1.0:
+                return norm.forward(resid, add, self.dtype, add_scale=scale)
+            return norm.forward(resid, add, self.dtype)
+
+        a = self.mixer.forward(normed(self.norm1, stream.pending, stream.pending_scale), ctx, cache)
+        if self.ffn is None:
+            return Stream(resid, a, pending_scale=self.scale)
+        m = self.ffn.forward(normed(self.norm2, a, self.scale), ctx)
+        return Stream(resid, m, pending_scale=self.scale)
 
 
 @register_block("branchnorm")
@@ -139,6 +173,8 @@ class BranchNormBlock(Block):
             raise RuntimeError("the stream carries a half-done norm of another block")
         rows_dtype = None if self.dtype == torch.float32 else self.dtype       # float32: the stream is its own rows
         x = stream.rows
+        if stream.pending is not None and stream.pending_scale != 1.0:
+            raise NotImplementedError("a branch with a factor is left to a block that norms its sublayers' outputs")
         if stream.pending is not None:        # a block of another arrangement left its last branch to be added
             x = kernels.rmsnorm_add(resid, stream.pending, None, 0.0, rows_dtype)
         if rows_dtype is None:

@@ -4,7 +4,8 @@
 float32 residual stream; with `sinusoid_base` b a sinusoidal position vector is added, entry 2i =
 sin(p b^(-2i / dim)), entry 2i + 1 = cos of the same angle, for the token's position p (float32) (reference: /root/reference/src/models/qwen3.rs:211-220,302-309).
 "lm_head": logits = h @ W^T in float32; W is the embedding table when the spec says `tied`
-(qwen3.rs:267-287,367-373); `softcap` c, if the spec gives one, makes them c * tanh(logits / c).
+(qwen3.rs:267-287,367-373); `scale` s, if the spec gives one, multiplies them; `softcap` c, if the spec
+gives one, then makes them c * tanh(logits / c).
 """
 from __future__ import annotations
 
@@ -64,6 +65,7 @@ class LMHead(Head):
         super().__init__(spec, dtype)
         self.tied = bool(spec.get("tied", False))
         self.softcap = float(spec.get("softcap") or 0.0)
+        self.scale = float(spec.get("scale") or 1.0)
         self.proj: Optional[Linear] = None
 
     @classmethod
@@ -85,4 +87,6 @@ class LMHead(Head):
         # the number of rows (thin or streaming up to 3, tiled up to 128, the library beyond), each
         # with its own order of sums, so they agree to rounding only
         logits = self.proj(h, out_dtype=torch.float32, skinny_rows=kernels.SKINNY_MAX_ROWS)
+        if self.scale != 1.0:
+            logits = kernels.scale_(logits, self.scale)
         return kernels.softcap_(logits, self.softcap) if self.softcap > 0 else logits

@@ -37,8 +37,8 @@ class RMSNorm(Norm):
         name = self.spec.get("name") or f"{prefix}.weight"
         self.weight = store.get(name, torch.float32, device).contiguous()
 
-    def forward(self, resid, add, out_dtype, rows=None, out=None):
-        return kernels.add_rmsnorm(resid, add, self.weight, self.eps, out_dtype, rows=rows, out=out)
+    def forward(self, resid, add, out_dtype, rows=None, out=None, add_scale: float = 1.0):
+        return kernels.add_rmsnorm(resid, add, self.weight, self.eps, out_dtype, rows=rows, out=out, y_scale=add_scale)
 
     def forward_branch(self, resid, y, rows_dtype):
         return kernels.rmsnorm_add(resid, y, self.weight, self.eps, rows_dtype)
