@@ -36,6 +36,9 @@ to 512 tokens, 256 new tokens each) at Qwen3-8B sizes: decode steps of 129 to 25
 bias, sublayer outputs normed, dense gelu or routed silu feed-forwards) beside Qwen3 at equal sizes
 (the same width, heads, head size, feed-forward width, window, vocabulary and number of layers): the
 prefill of one prompt and a decode step at batch 8, one JSON line with both.
+`--design lilalorn[:SIZE]` times the Lilalorn family (layers of softmax attention beside retention, and of
+gated linear attention, in turn; experts without a gate and a shared one) beside the closest family there
+is, Mufenex with routed experts and no window, at equal sizes.
 """
 from __future__ import annotations
 
@@ -79,7 +82,9 @@ DESIGN_SIZES = {
     "4k": dict(width=4096, heads=32, kv_heads=8, dim=128, vdim=128, ff=12288, window=2048, experts=0, top=0),
     "4k-moe": dict(width=4096, heads=32, kv_heads=8, dim=128, vdim=128, ff=12288, window=2048, experts=8, top=2),
     "2k-v": dict(width=2048, heads=16, kv_heads=4, dim=64, vdim=128, ff=8192, window=512, experts=16, top=2),
+    "1k-moe": dict(width=1024, heads=16, kv_heads=8, dim=128, vdim=128, ff=3072, window=1024, experts=8, top=2),
 }
+LILALORN_SIZES = ("1k-moe", "4k-moe", "2k-v")      # the sizes with experts: every Lilalorn layer has them
 DESIGN_VOCAB = 32000
 MODELS = {"0.6b": QWEN3_0_6B, "8b": QWEN3_8B, "14b": QWEN3_14B, "32b": QWEN3_32B}
 CONTEXT = 4096
@@ -217,21 +222,26 @@ def product(spec: str, dev="cuda:0") -> int:
 
 def design_compare(spec: str, layers, steps: int, warmup: int, batch: int, context: int, prefill_tokens: int,
                    family: str = "both", only: str = "all") -> int:
-    """Mufenex beside Qwen3 at equal sizes: ms of the prefill of one prompt and of a decode step."""
+    """Mufenex beside Qwen3, or Lilalorn beside Mufenex, at equal sizes: ms of the prefill of one prompt and of a
+    decode step."""
     import torch
     from xinfer_amd.engine import ModelRunner, StepEntry, build_model
     from xinfer_amd.models import config_from_dict
     from xinfer_amd.sampling import Sampler
     from xinfer_amd.weights.random_init import random_store_for
     name, _, size = spec.partition(":")
-    if name != "mufenex" or (size and size not in DESIGN_SIZES):
-        print(f"bench.py: --design mufenex[:{'|'.join(DESIGN_SIZES)}]")
+    if name not in ("mufenex", "lilalorn") or (size and size not in (DESIGN_SIZES if name == "mufenex" else LILALORN_SIZES)):
+        print(f"bench.py: --design mufenex[:{'|'.join(DESIGN_SIZES)}] or lilalorn[:{'|'.join(LILALORN_SIZES)}]")
+        return 2
+    beside = "qwen3" if name == "mufenex" else "mufenex"
+    if family not in ("both", name, beside):
+        print(f"bench.py: --family both, {name} or {beside} with --design {name}")
         return 2
     dev, page = "cuda:0", 64
     layers = layers or 4
     sampler = Sampler(dev)
     gen = torch.Generator().manual_seed(3)
-    out = {"metric": "Mufenex beside Qwen3 at equal sizes, bf16", "unit": "ms", "layers": layers, "batch": batch,
+    out = {"metric": f"{name.capitalize()} beside {beside.capitalize()} at equal sizes, bf16", "unit": "ms", "layers": layers, "batch": batch,
            "context": context, "prefill_tokens": prefill_tokens, "data": "synthetic: seeded random weights and token ids",
            "sizes": {}}
 
@@ -246,7 +256,25 @@ def design_compare(spec: str, layers, steps: int, warmup: int, batch: int, conte
         qwen3 = dict(QWEN3_8B, hidden_size=z["width"], intermediate_size=z["ff"], num_hidden_layers=layers,
                      num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"], head_dim=z["dim"],
                      vocab_size=DESIGN_VOCAB, sliding_window=z["window"], max_position_embeddings=2 * context)
-        return {"mufenex": mufenex, "qwen3": qwen3}
+        if name == "mufenex":
+            return {"mufenex": mufenex, "qwen3": qwen3}
+        # Lilalorn: layers of attention beside retention and of gated linear attention in turn; the states' heads are a
+        # quarter as many as the query heads, keys as wide as the attention's and values twice that
+        mixer.pop("mask")
+        mixer["v_mix"] = False
+        sh = max(1, z["heads"] // 4)
+        moe = {"kind": "moe", "expert": {"ff": z["ff"] // z["top"]}, "router": {"experts": z["experts"], "top": z["top"]},
+               "shared": {"ff": z["ff"] // z["top"]}}
+        par = {"type": "parallel", "mlp": moe, "mixer": {
+            "left": dict(heads=z["heads"], kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["vdim"], scale=z["dim"] ** -0.5,
+                         rot=dict(dims=z["dim"], base=500000.0, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192))),
+            "right": dict(heads=sh, dim=z["dim"], vdim=2 * z["dim"], decay=[1.0 - 2.0 ** -(5 + h % 6) for h in range(sh)]),
+            "left_scale": 0.6, "right_scale": 0.5}}
+        gla = {"type": "gla", "mlp": moe, "mixer": dict(heads=sh, dim=z["dim"], vdim=2 * z["dim"], tau=16.0)}
+        lilalorn = {"architecture": "Lilalorn", "vocab": DESIGN_VOCAB, "width": z["width"], "norm": {"eps": 1e-6},
+                    "residual_mult": 0.7, "logit_scale": 0.5, "max_positions": 2 * context,
+                    "layers": [par if i % 2 == 0 else gla for i in range(layers)]}
+        return {"lilalorn": lilalorn, "mufenex": mufenex}
 
     def time_model(raw):
         _, cfg = config_from_dict(raw)
@@ -305,12 +333,12 @@ def design_compare(spec: str, layers, steps: int, warmup: int, batch: int, conte
             res.update({"prefill_ms": round(best * 1e3, 3), "prefill_tok_s": round(prefill_tokens / best, 1)})
         return res
 
-    for key in ([size] if size else list(DESIGN_SIZES)):
+    for key in ([size] if size else list(DESIGN_SIZES if name == "mufenex" else LILALORN_SIZES)):
         z = DESIGN_SIZES[key]
         res = {k: time_model(raw) for k, raw in configs(z).items() if family in ("both", k)}
         for what in ("prefill", "decode"):
-            if family == "both" and f"{what}_ms" in res["mufenex"]:
-                res[f"ratio_{what}"] = round(res["mufenex"][f"{what}_ms"] / res["qwen3"][f"{what}_ms"], 3)
+            if family == "both" and f"{what}_ms" in res[name]:
+                res[f"ratio_{what}"] = round(res[name][f"{what}_ms"] / res[beside][f"{what}_ms"], 3)
         out["sizes"][key] = dict(z, **res)
         print(f"[bench] {key}: {res}", file=sys.stderr, flush=True)
     print(json.dumps(out), flush=True)
@@ -376,10 +404,10 @@ def main() -> int:
                     help="serving workloads: read every step's tokens on the host before the next step is planned")
     ap.add_argument("--product", default=None, metavar="M,N,K[,slices[,shape]]",
                     help="time one bfloat16 product alone in the many-row tiled kernel and in the vendor library")
-    ap.add_argument("--design", default=None, metavar="mufenex[:SIZE]",
-                    help="time another model family beside Qwen3 at equal sizes (a line of its own; --layers, --steps, "
+    ap.add_argument("--design", default=None, metavar="mufenex[:SIZE]|lilalorn[:SIZE]",
+                    help="time another model family beside its closest one (Mufenex beside Qwen3, Lilalorn beside Mufenex) at equal sizes (a line of its own; --layers, --steps, "
                          "--warmup, --batch, --context, --prefill-tokens and --only apply)")
-    ap.add_argument("--family", choices=["both", "mufenex", "qwen3"], default="both",
+    ap.add_argument("--family", choices=["both", "lilalorn", "mufenex", "qwen3"], default="both",
                     help="--design: time one of the two families only (for profiling)")
     ap.add_argument("--peaks", action="store_true",
                     help="also measure what this card reaches on a read-only stream of 4 GiB and on one square "

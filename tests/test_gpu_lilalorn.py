@@ -51,15 +51,19 @@ def _decays(T, H, dk, z, bias, decay, tau):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("chunk", [0, 16])
 @pytest.mark.parametrize("per_token", [False, True])
 @pytest.mark.parametrize("H,dk,dv", [(2, 16, 24), (3, 10, 6), (1, 192, 64), (2, 128, 256), (1, 7, 70), (1, 256, 8)])
-def test_state_walk_of_unequal_requests_in_portions(H, dk, dv, per_token, dtype):
+def test_state_walk_of_unequal_requests_in_portions(H, dk, dv, per_token, chunk, dtype, monkeypatch):
     """Three requests of unequal length in one batch, in slots that are not in order, cut into portions of several
-    sizes down to one token: every portion starts from the state the one before left in the slot."""
+    sizes down to one token: every portion starts from the state the one before left in the slot.  With `chunk`
+    the long portions are walked in chunks of 16 tokens side by side (a last chunk of one token, a chunked portion
+    beside single tokens), the short ones in one piece."""
     from xinfer_amd import kernels
+    monkeypatch.setattr(kernels, "SCAN_CHUNK", chunk)
     dt, tau = TD[dtype], 4.0
     lens = [37, 5, 70]
-    cuts = {0: [2, 30, 1, 4], 1: [5], 2: [1, 1, 2, 64, 2]}
+    cuts = {0: [2, 33, 1, 1], 1: [5], 2: [1, 1, 2, 64, 2]}
     slots = [3, 0, 2]
     data = [_scan_inputs(n, H, dk, dv, dt, 10 * i + H, per_token) for i, n in enumerate(lens)]
     want = []
@@ -86,7 +90,8 @@ def test_state_walk_of_unequal_requests_in_portions(H, dk, dv, per_token, dtype)
         o = kernels.linear_scan(q, k, v, state, torch.tensor([slots[b] for b in who], device=DEV),
                                 torch.tensor(cu, dtype=torch.int32, device=DEV), H, dk, dv, z=zz, tau=tau,
                                 z_bias=data[0][5].to(DEV) if per_token else None,
-                                head_decay=None if per_token else data[0][6].to(DEV), q_scale=0.5, k_scale=0.25)
+                                head_decay=None if per_token else data[0][6].to(DEV), q_scale=0.5, k_scale=0.25,
+                                q_lens=[n for _, _, n in rows] if chunk else None, plan_cache={} if step % 2 else None)
         for i, (b, a, n) in enumerate(rows):
             got[b].append(o[cu[i]:cu[i + 1]].cpu())
     assert torch.all(state[1] == 7.0) and torch.all(state[4] == 7.0)        # other slots are left alone
@@ -94,6 +99,16 @@ def test_state_walk_of_unequal_requests_in_portions(H, dk, dv, per_token, dtype)
         g = torch.cat(got[b]).double()
         assert g.shape == want[b].shape
         assert (g - want[b]).abs().max() < 2e-5 * want[b].abs().max(), (b, float((g - want[b]).abs().max()))
+
+
+def test_the_cutting_of_long_portions():
+    from xinfer_amd import kernels
+    whole, long, chunks = kernels.scan_chunk_plan([1, 130, 64, 128, 300, 127], 64)
+    assert whole == [0, 2, 5] and long == [(1, 0, 3), (3, 3, 2), (4, 5, 5)]
+    assert chunks == [(0, 64), (64, 64), (128, 2), (0, 64), (64, 64), (0, 64), (64, 64), (128, 64), (192, 64), (256, 44)]
+    assert kernels.scan_chunk_plan([500, 3], 0) == ([0, 1], [], [])
+    _, long, chunks = kernels.scan_chunk_plan([100_000], 64)           # no more chunks than their states have room for
+    assert len(chunks) <= kernels.SCAN_CHUNKS_MOST and sum(n for _, n in chunks) == 100_000
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -124,7 +139,7 @@ def test_state_keeps_a_far_key(decay, far, dtype):
     for a, b in [(0, 257), (257, T - 5)] + [(t, t + 1) for t in range(T - 5, T)]:
         cu = torch.tensor([0, b - a], dtype=torch.int32, device=DEV)
         outs.append(kernels.linear_scan(q[a:b].to(DEV), k[a:b].to(DEV), v[a:b].to(DEV), state, slot, cu, H, dk, dv,
-                                        head_decay=torch.full((H,), decay, device=DEV)).cpu())
+                                        head_decay=torch.full((H,), decay, device=DEV), q_lens=[b - a]).cpu())
     got = torch.cat(outs).double()
     assert (got - want).abs().max() < 3e-5 * want.abs().max()
 
@@ -411,6 +426,17 @@ def test_mixed_batches_with_pages_and_slots_used_again(name, dtype, dirs):
     finds no state of the one before."""
     for seed in (1, 2):
         _run(name, dtype, dirs, harness.trace_mixed(_requests(name), seed, max_live=3), f"mixed {seed}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "O"])
+def test_short_chunks_of_the_states_walk(name, dtype, dirs, monkeypatch):
+    """Portions from 32 tokens on are walked in chunks of 16: whole prompts, portions and mixed batches again."""
+    from xinfer_amd import kernels
+    monkeypatch.setattr(kernels, "SCAN_CHUNK", 16)
+    _run(name, dtype, dirs, harness.trace_whole(_requests(name)), "whole, chunks of 16")
+    _run(name, dtype, dirs, harness.trace_portions(_requests(name), sizes=(33, 2, 47, 32, 5)), "portions, chunks of 16")
+    _run(name, dtype, dirs, harness.trace_mixed(_requests(name), 3, max_live=3, sizes=(40, 2, 35, 64)), "mixed, chunks of 16")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

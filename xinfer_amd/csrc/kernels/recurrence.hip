@@ -11,12 +11,20 @@
 // q, k and v are columns of a packed projection (a row stride and a column offset each); q and k are
 // multiplied by `q_scale` / `k_scale` in float32 as they are read.
 //
-// `linear_scan_kernel`: one workgroup per (request, head, 64 value columns) walks the request's tokens of
-// this step in order, from the state its slot holds, and leaves the new state there: the result does not
-// depend on how a prompt was cut into steps or on what else is in the batch, bit for bit.  Lane l owns
-// value column l of the tile, wave w the key channels w, w + 4, ..; a thread keeps its RPT state elements
-// in registers for the whole walk.  A token costs one barrier: q, k and the decay of the next token are
-// fetched while this one is worked on.
+// `linear_scan_kernel`: one workgroup per (item, head, 64 value columns) walks the item's tokens in order,
+// from a state it is told to start from, and may leave the new state somewhere.  Lane l owns value column l
+// of the tile, wave w the key channels w, w + 4, ..; a thread keeps its RPT state elements in registers for
+// the whole walk.  A token costs one barrier: q, k and the decay of the next token are fetched while this
+// one is worked on.  An item is a request's tokens of this step (from the state in its slot, back into it:
+// steps of single tokens and short portions; what a token gets then does not depend on how the prompt was
+// cut, bit for bit), or one chunk of a long portion:
+//
+// A long portion is cut into chunks that are walked side by side, in three launches.  (1) every chunk but a
+// portion's last, from a zero state and without results: its own share U_c = sum_s (prod_{r > s} a_r) k_s v_s^T
+// and the product D_c of its decays; (2) `chunk_carry_kernel`, element by element: the state S_c each chunk
+// starts from, S_0 = the slot's, S_{c+1} = D_c S_c + U_c; (3) every chunk from its S_c, with results, the
+// portion's last chunk leaving its state in the slot.  Twice the arithmetic of one walk, in a chain a chunk
+// long instead of a portion long; all of it float32, so the three launches and the one walk agree to rounding.
 //
 // `head_norm_gate_kernel`: what follows the state in both mixers: each head's o divided by its root mean
 // square over dv (eps inside the root), times a weight [dv] shared by the heads (or none), times silu(g),
@@ -40,22 +48,26 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
     const T* __restrict__ q, long long q_stride, const T* __restrict__ k, long long k_stride, const T* __restrict__ v,
     long long v_stride, const float* __restrict__ z, const float* __restrict__ z_bias, float inv_tau,
     const float* __restrict__ head_decay,
-    float* __restrict__ state, long long slot_stride, const long long* __restrict__ state_slots,
-    const int* __restrict__ cu_q, float* __restrict__ out, int H, int dk, int dv, float q_scale, float k_scale) {
+    const float* __restrict__ state_in, long long in_stride, const long long* __restrict__ in_idx,
+    float* __restrict__ state_out, long long out_stride, const long long* __restrict__ out_idx,
+    const int* __restrict__ first, const int* __restrict__ last, float* __restrict__ out, float* __restrict__ decay_out,
+    int H, int dk, int dv, float q_scale, float k_scale) {
   __shared__ float qs[2][kScanWaves * 64], ks[2][kScanWaves * 64], as[2][kScanWaves * 64];
   __shared__ float part[2][kScanWaves][kScanCols];
   const int b = blockIdx.x, h = blockIdx.y, j = blockIdx.z * kScanCols + (threadIdx.x & 63);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int t0 = cu_q[b], t1 = cu_q[b + 1];
+  const int t0 = first[b], t1 = last[b];
   if (t1 <= t0) return;
   const bool col = j < dv;
-  float* S = state + (size_t)state_slots[b] * slot_stride + (size_t)h * dk * dv;
+  const long long from = in_idx ? in_idx[b] : -1, to = out_idx ? out_idx[b] : -1;      // negative: from zeros / kept nowhere
+  const float* S = state_in + (size_t)(from < 0 ? 0 : from) * in_stride + (size_t)h * dk * dv;
   float s[RPT];
 #pragma unroll
   for (int r = 0; r < RPT; ++r) {
     const int i = wave + kScanWaves * r;
-    s[r] = (col && i < dk) ? S[(size_t)i * dv + j] : 0.f;
+    s[r] = (from >= 0 && col && i < dk) ? S[(size_t)i * dv + j] : 0.f;
   }
+  float all_decays = 1.f;               // of channel c, over the item's tokens
   const int c = threadIdx.x;            // the channel this thread fetches for the workgroup
   const float hd = head_decay ? head_decay[h] : 0.f;
   const float zb = (z_bias && c < dk) ? z_bias[h * dk + c] : 0.f;
@@ -76,6 +88,7 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
   __syncthreads();
   for (int t = t0; t < t1; ++t) {
     const int cur = (t - t0) & 1;
+    all_decays *= fa;
     if (t + 1 < t1) fetch(t + 1, fq, fk, fa);
     const float vj = col ? to_float(v[(size_t)t * v_stride + h * dv + j]) : 0.f;
     float acc = 0.f;
@@ -87,20 +100,46 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
         acc = fmaf(s[r], qs[cur][i], acc);
       }
     }
-    part[cur][wave][lane] = acc;
+    if (out) part[cur][wave][lane] = acc;
     if (t + 1 < t1 && c < dk) {
       qs[cur ^ 1][c] = fq;
       ks[cur ^ 1][c] = fk;
       as[cur ^ 1][c] = fa;
     }
     __syncthreads();
-    if (wave == 0 && col)
+    if (out && wave == 0 && col)
       out[((size_t)t * H + h) * dv + j] = (part[cur][0][lane] + part[cur][1][lane]) + (part[cur][2][lane] + part[cur][3][lane]);
   }
+  if (to >= 0) {
+    float* D = state_out + (size_t)to * out_stride + (size_t)h * dk * dv;
 #pragma unroll
-  for (int r = 0; r < RPT; ++r) {
-    const int i = wave + kScanWaves * r;
-    if (col && i < dk) S[(size_t)i * dv + j] = s[r];
+    for (int r = 0; r < RPT; ++r) {
+      const int i = wave + kScanWaves * r;
+      if (col && i < dk) D[(size_t)i * dv + j] = s[r];
+    }
+  }
+  if (decay_out && blockIdx.z == 0 && c < dk) decay_out[((size_t)b * H + h) * dk + c] = all_decays;
+}
+
+// The states that the chunks of long portions start from.  Portion p has n[p] chunks, numbered from c0[p]:
+// starts[c0] = the slot's state, starts[c + 1] = decays[c] (per key channel) * starts[c] + shares[c].
+// One thread an element of the state, one grid row a portion.
+__global__ __launch_bounds__(256) void chunk_carry_kernel(const float* __restrict__ state, long long slot_stride,
+                                                          const long long* __restrict__ slots, const int* __restrict__ c0,
+                                                          const int* __restrict__ n, const float* __restrict__ shares,
+                                                          const float* __restrict__ decays, float* __restrict__ starts,
+                                                          int H, int dk, int dv) {
+  const int p = blockIdx.y;
+  const size_t per = (size_t)H * dk * dv;
+  const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= per) return;
+  const size_t hi = e / dv;                 // (head, key channel)
+  float s = state[(size_t)slots[p] * slot_stride + e];
+  const int first = c0[p], count = n[p];
+  for (int c = 0; c < count; ++c) {
+    const size_t at = (size_t)(first + c);
+    starts[at * per + e] = s;
+    if (c + 1 < count) s = fmaf(decays[at * H * dk + hi], s, shares[at * per + e]);
   }
 }
 
@@ -134,26 +173,33 @@ using namespace xi;
 extern "C" {
 
 // q, k [T, .] with H dk columns from the given pointers, v with H dv, rows `*_stride` elements apart, in `dtype`;
-// z float32 [T, H dk] (z_bias float32 [H dk] or null) or null (then head_decay float32 [H]); state float32, slot s at state + s * slot_stride,
-// [H, dk, dv]; state_slots int64 [B]; cu_q int32 [B + 1]; out float32 [T, H, dv].
+// z float32 [T, H dk] (z_bias float32 [H dk] or null) or null (then head_decay float32 [H]).  Item w walks tokens
+// first[w] .. last[w] - 1 from the state state_in + in_idx[w] * in_stride ([H, dk, dv] float32; in_idx null or a
+// negative entry: from zeros) and leaves its last state at state_out + out_idx[w] * out_stride (null or negative:
+// nowhere); out float32 [T, H, dv] or null (no results); decay_out float32 [items, H, dk] or null: the product of
+// each channel's decays over the item.
 int xi_linear_scan(const void* q, long long q_stride, const void* k, long long k_stride, const void* v, long long v_stride,
-                   int dtype, const float* z, const float* z_bias, float tau, const float* head_decay, float* state, long long slot_stride,
-                   const long long* state_slots, const int* cu_q, float* out, int n_seqs, int H, int dk, int dv,
-                   float q_scale, float k_scale, hipStream_t stream) {
-  XI_CHECK(n_seqs >= 0 && H > 0 && dk > 0 && dv > 0, "linear_scan: bad sizes B=%d H=%d dk=%d dv=%d", n_seqs, H, dk, dv);
+                   int dtype, const float* z, const float* z_bias, float tau, const float* head_decay, const float* state_in,
+                   long long in_stride, const long long* in_idx, float* state_out, long long out_stride,
+                   const long long* out_idx, const int* first, const int* last, float* out, float* decay_out, int n_items, int H,
+                   int dk, int dv, float q_scale, float k_scale, hipStream_t stream) {
+  XI_CHECK(n_items >= 0 && H > 0 && dk > 0 && dv > 0, "linear_scan: bad sizes items=%d H=%d dk=%d dv=%d", n_items, H, dk, dv);
   XI_CHECK(dk <= kScanWaves * 64, "linear_scan: key heads of up to %d channels, not %d", kScanWaves * 64, dk);
   XI_CHECK((z != nullptr) != (head_decay != nullptr), "linear_scan: a decay per token or a decay per head, one of them");
   XI_CHECK(z == nullptr || tau > 0.f, "linear_scan: tau must be positive");
-  XI_CHECK(slot_stride >= (long long)H * dk * dv, "linear_scan: a state slot is too small");
-  if (n_seqs == 0) return 0;
-  dim3 grid((unsigned)n_seqs, (unsigned)H, (unsigned)((dv + kScanCols - 1) / kScanCols));
+  XI_CHECK((in_idx == nullptr || (state_in && in_stride >= (long long)H * dk * dv)) &&
+               (out_idx == nullptr || (state_out && out_stride >= (long long)H * dk * dv)),
+           "linear_scan: states need a place of at least H dk dv floats each");
+  XI_CHECK(first && last, "linear_scan: the items' token ranges are missing");
+  if (n_items == 0) return 0;
+  dim3 grid((unsigned)n_items, (unsigned)H, (unsigned)((dv + kScanCols - 1) / kScanCols));
   XI_CHECK(grid.y <= 65535u && grid.z <= 65535u, "linear_scan: too many heads or value columns");
   const float inv_tau = z ? 1.f / tau : 0.f;
   const int rpt = (dk + kScanWaves - 1) / kScanWaves;
-#define XI_SCAN(TT, R)                                                                                                   \
-  linear_scan_kernel<TT, R><<<grid, kScanWaves * kWave, 0, stream>>>(                                                    \
-      (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v, v_stride, z, z_bias, inv_tau, head_decay, state, slot_stride, \
-      state_slots, cu_q, out, H, dk, dv, q_scale, k_scale)
+#define XI_SCAN(TT, R)                                                                                                        \
+  linear_scan_kernel<TT, R><<<grid, kScanWaves * kWave, 0, stream>>>(                                                         \
+      (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v, v_stride, z, z_bias, inv_tau, head_decay, state_in, in_stride, \
+      in_idx, state_out, out_stride, out_idx, first, last, out, decay_out, H, dk, dv, q_scale, k_scale)
 #define XI_SCAN_T(TT)            \
   do {                           \
     if (rpt <= 8) XI_SCAN(TT, 8); \
@@ -167,6 +213,22 @@ int xi_linear_scan(const void* q, long long q_stride, const void* k, long long k
 #undef XI_SCAN_T
 #undef XI_SCAN
   XI_LAUNCH_CHECK("linear_scan");
+  return 0;
+}
+
+// state float32, slot s at state + s * slot_stride; slots int64 [P]; c0, n int32 [P]; shares, starts float32
+// [chunks, H, dk, dv]; decays float32 [chunks, H, dk].
+int xi_chunk_carry(const float* state, long long slot_stride, const long long* slots, const int* c0, const int* n,
+                   const float* shares, const float* decays, float* starts, int n_portions, int H, int dk, int dv,
+                   hipStream_t stream) {
+  XI_CHECK(n_portions >= 0 && H > 0 && dk > 0 && dv > 0, "chunk_carry: bad sizes portions=%d H=%d dk=%d dv=%d", n_portions, H, dk, dv);
+  XI_CHECK(slot_stride >= (long long)H * dk * dv, "chunk_carry: a state slot is too small");
+  if (n_portions == 0) return 0;
+  const size_t per = (size_t)H * dk * dv;
+  dim3 grid((unsigned)((per + 255) / 256), (unsigned)n_portions);
+  XI_CHECK(grid.y <= 65535u, "chunk_carry: too many portions");
+  chunk_carry_kernel<<<grid, 256, 0, stream>>>(state, slot_stride, slots, c0, n, shares, decays, starts, H, dk, dv);
+  XI_LAUNCH_CHECK("chunk_carry");
   return 0;
 }
 

@@ -253,16 +253,54 @@ def _columns(t: torch.Tensor, width: int, what: str):
     return int(t.stride(0)) if t.shape[0] > 1 else width
 
 
+SCAN_CHUNK = 64           # tokens of a chunk of a long portion (see `linear_scan`); 0: every portion is walked in one piece
+SCAN_CHUNKS_MOST = 512    # chunks of a step at most (their states are kept side by side): longer steps get longer chunks
+
+
+def scan_chunk_plan(q_lens, chunk: Optional[int] = None):
+    """How a step's portions are walked by `linear_scan`: (whole, long, chunks) with `whole` the batch rows walked in
+    one piece (single tokens and portions of less than two chunks) and, for the others, `long` = [(row, first chunk,
+    number of chunks)] and `chunks` = [(first token within the portion, tokens)] in the order of their numbers."""
+    chunk = SCAN_CHUNK if chunk is None else int(chunk)
+    total = sum(int(n) for n in q_lens)
+    if chunk > 0 and total > chunk * SCAN_CHUNKS_MOST:
+        chunk = -(-total // SCAN_CHUNKS_MOST // 16) * 16
+    whole, long, chunks = [], [], []
+    for b, n in enumerate(q_lens):
+        n = int(n)
+        if chunk <= 0 or n < 2 * chunk:
+            whole.append(b)
+            continue
+        count = -(-n // chunk)
+        long.append((b, len(chunks), count))
+        chunks += [(c * chunk, min(chunk, n - c * chunk)) for c in range(count)]
+    return whole, long, chunks
+
+
+def _scan_launch(q, k, v, qs, ks, vs, z, z_bias, tau, head_decay, state_in, in_stride, in_idx, state_out, out_stride, out_idx,
+                 first, last, out, decay_out, items, H, dk, dv, q_scale, k_scale):
+    _ok(lib().xi_linear_scan(_p(q), ctypes.c_longlong(qs), _p(k), ctypes.c_longlong(ks), _p(v), ctypes.c_longlong(vs),
+                             _code(q, "linear_scan"), _p(z), _p(z_bias), ctypes.c_float(tau), _p(head_decay), _p(state_in),
+                             ctypes.c_longlong(in_stride), _p(in_idx), _p(state_out), ctypes.c_longlong(out_stride),
+                             _p(out_idx), ctypes.c_void_p(first), ctypes.c_void_p(last), _p(out), _p(decay_out), int(items),
+                             H, dk, dv, ctypes.c_float(q_scale), ctypes.c_float(k_scale), _stream()))
+
+
 def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.Tensor, state_slots: torch.Tensor,
                 cu_q: torch.Tensor, heads: int, key_dim: int, value_dim: int, z: Optional[torch.Tensor] = None,
                 tau: float = 1.0, head_decay: Optional[torch.Tensor] = None, q_scale: float = 1.0,
-                k_scale: float = 1.0, z_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+                k_scale: float = 1.0, z_bias: Optional[torch.Tensor] = None, q_lens=None, plan_cache=None) -> torch.Tensor:
     """Linear attention with a decaying float32 state per request and head, S <- diag(a) S + k v^T, o = S^T q,
     token by token from the state each request's slot holds (left there afterwards).  q, k [T, H dk] and
     v [T, H dv] may be column ranges of a packed projection.  The decay: `z` float32 [T, H dk], `z_bias`
     float32 [H dk] (or None) and `tau` (a = sigmoid(z + bias)^(1 / tau) per token and key channel) or `head_decay` float32 [H] (a constant per head).
     state float32 [slots, H, dk, dv] (slots may be strided); state_slots int64 [B]; cu_q int32 [B + 1].
-    Returns o float32 [T, H, dv]."""
+    Returns o float32 [T, H, dv].
+    `q_lens` (the host's copy of the portions' lengths; None: nothing of the step is read on the host, as a step
+    of single tokens wants it): portions of two chunks and more (`SCAN_CHUNK`) are cut into chunks that are walked
+    side by side in three launches (each chunk's own share from a zero state; the states the chunks start from,
+    one after the other; the chunks' results), the others in one piece.  `plan_cache`: a dict of the step in which
+    the index arrays of this cutting are kept for the next layer."""
     H, dk, dv = int(heads), int(key_dim), int(value_dim)
     T = q.shape[0]
     qs, ks, vs = _columns(q, H * dk, "linear_scan: q"), _columns(k, H * dk, "linear_scan: k"), _columns(v, H * dv, "linear_scan: v")
@@ -290,11 +328,59 @@ def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.
     B = state_slots.shape[0]
     if cu_q.shape != (B + 1,) or dk > 256:
         raise KernelError("linear_scan: cu_q must be [B + 1]; key heads of up to 256 channels")
+    if q_lens is not None and (len(q_lens) != B or sum(int(n) for n in q_lens) != T):
+        raise KernelError("linear_scan: the portions' lengths do not add up to the step's tokens")
     out = torch.empty((T, H, dv), dtype=torch.float32, device=q.device)
-    _ok(lib().xi_linear_scan(_p(q), ctypes.c_longlong(qs), _p(k), ctypes.c_longlong(ks), _p(v), ctypes.c_longlong(vs),
-                             _code(q, "linear_scan"), _p(z), _p(z_bias), ctypes.c_float(tau), _p(head_decay), _p(state),
-                             ctypes.c_longlong(int(state.stride(0)) if state.shape[0] > 1 else H * dk * dv), _p(state_slots),
-                             _p(cu_q), _p(out), B, H, dk, dv, ctypes.c_float(q_scale), ctypes.c_float(k_scale), _stream()))
+    slot_stride = int(state.stride(0)) if state.shape[0] > 1 else H * dk * dv
+    common = (q, k, v, qs, ks, vs, z, z_bias, tau, head_decay)
+    whole, long, chunks = scan_chunk_plan(q_lens) if q_lens is not None else (None, [], [])
+    if not long:            # every request in one piece, straight from the step's own arrays
+        _scan_launch(*common, state, slot_stride, state_slots, state, slot_stride, state_slots, cu_q.data_ptr(),
+                     cu_q.data_ptr() + 4, out, None, B, H, dk, dv, q_scale, k_scale)
+        return out
+    key = ("linear_scan_plan", SCAN_CHUNK)
+    plan = plan_cache.get(key) if plan_cache is not None else None
+    if plan is None:             # the same for every layer of the step: made once
+        starts = [0]
+        for n in q_lens:
+            starts.append(starts[-1] + int(n))
+        C, L, W = len(chunks), len(long), len(whole)
+        first, last, hands_on = [0] * C, [0] * C, [False] * C
+        for b, c0, count in long:
+            for c in range(count):
+                first[c0 + c] = starts[b] + chunks[c0 + c][0]
+                last[c0 + c] = first[c0 + c] + chunks[c0 + c][1]
+                hands_on[c0 + c] = c + 1 < count          # a portion's last chunk hands no share on
+        i32 = torch.tensor(first + last
+                           + [f if h else 0 for f, h in zip(first, hands_on)] + [l if h else 0 for l, h in zip(last, hands_on)]
+                           + [c0 for _, c0, _ in long] + [n for _, _, n in long]
+                           + [starts[b] for b in whole] + [starts[b + 1] for b in whole], dtype=torch.int32).to(q.device)
+        i64 = torch.tensor([c if h else -1 for c, h in enumerate(hands_on)] + list(range(C)) + [-1] * C
+                           + [b for b, _, _ in long] + [c0 + n - 1 for _, c0, n in long] + whole, dtype=torch.int64).to(q.device)
+        long_slots = state_slots.index_select(0, i64[3 * C:3 * C + L])
+        keep = i64[2 * C:3 * C]         # where launch 3 leaves a chunk's last state: a portion's last chunk in the slot
+        keep.index_copy_(0, i64[3 * C + L:3 * C + 2 * L], long_slots)
+        slots_w = state_slots.index_select(0, i64[3 * C + 2 * L:]) if W else None
+        plan = dict(C=C, L=L, W=W, first=i32[:C], last=i32[C:2 * C], first1=i32[2 * C:3 * C], last1=i32[3 * C:4 * C],
+                    c0=i32[4 * C:4 * C + L], n=i32[4 * C + L:4 * C + 2 * L], wfirst=i32[4 * C + 2 * L:4 * C + 2 * L + W],
+                    wlast=i32[4 * C + 2 * L + W:], share_to=i64[:C], every=i64[C:2 * C], keep=keep, long_slots=long_slots,
+                    slots_w=slots_w)
+        if plan_cache is not None:
+            plan_cache[key] = plan
+    P = plan
+    C, per = P["C"], H * dk * dv
+    shares = torch.empty((C, H, dk, dv), dtype=torch.float32, device=q.device)
+    begins = torch.empty((C, H, dk, dv), dtype=torch.float32, device=q.device)
+    decays = torch.empty((C, H, dk), dtype=torch.float32, device=q.device)
+    _scan_launch(*common, None, 0, None, shares, per, P["share_to"], P["first1"].data_ptr(), P["last1"].data_ptr(), None, decays,
+                 C, H, dk, dv, q_scale, k_scale)
+    _ok(lib().xi_chunk_carry(_p(state), ctypes.c_longlong(slot_stride), _p(P["long_slots"]), _p(P["c0"]), _p(P["n"]), _p(shares),
+                             _p(decays), _p(begins), P["L"], H, dk, dv, _stream()))
+    _scan_launch(*common, begins, per, P["every"], state, slot_stride, P["keep"], P["first"].data_ptr(), P["last"].data_ptr(), out,
+                 None, C, H, dk, dv, q_scale, k_scale)
+    if P["W"]:
+        _scan_launch(*common, state, slot_stride, P["slots_w"], state, slot_stride, P["slots_w"], P["wfirst"].data_ptr(),
+                     P["wlast"].data_ptr(), out, None, P["W"], H, dk, dv, q_scale, k_scale)
     return out
 
 

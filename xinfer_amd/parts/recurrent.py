@@ -83,6 +83,15 @@ class _DecayingState(Mixer):
         return p[:, :a], p[:, a:2 * a], p[:, 2 * a:2 * a + b], p[:, 2 * a + b:2 * a + 2 * b]
 
     @staticmethod
+    def _cutting(ctx: StepContext):
+        """What the state's kernel may know of the step on the host: nothing in a step of single tokens (which may be
+        recorded), the portions' lengths otherwise (long portions are then walked chunk by chunk, side by side)."""
+        if ctx.max_q_len <= 1 or not ctx.cu_q_host:
+            return {}
+        cu = ctx.cu_q_host
+        return dict(q_lens=[cu[b + 1] - cu[b] for b in range(ctx.num_seqs)], plan_cache=ctx.scratch)
+
+    @staticmethod
     def _state(cache: LayerCache) -> torch.Tensor:
         if cache.state is None:
             raise RuntimeError("a mixer with a decaying state was given no state slots")
@@ -125,7 +134,7 @@ class GatedLinearAttention(_DecayingState):
         # the decay's logits leave the second product in float32; their bias is added where they are read
         z = self.a2(self.a1(x, out_dtype=self.dtype), out_dtype=torch.float32)
         o = kernels.linear_scan(q, k, v, self._state(cache), ctx.state_slots, ctx.cu_q, self.heads, self.dk, self.dv,
-                                z=z, z_bias=self.a2_bias, tau=self.tau, q_scale=self.q_scale)
+                                z=z, z_bias=self.a2_bias, tau=self.tau, q_scale=self.q_scale, **self._cutting(ctx))
         return self.o(kernels.head_norm_gate(o, self.norm_w, self.eps, g, self.dtype), out_dtype=self.dtype)
 
 
@@ -151,5 +160,5 @@ class Retention(_DecayingState):
         p = self.proj(x, out_dtype=self.dtype)
         q, k, v, g = self._split(p)
         o = kernels.linear_scan(q, k, v, self._state(cache), ctx.state_slots, ctx.cu_q, self.heads, self.dk, self.dv,
-                                head_decay=self.decay, k_scale=self.k_scale)
+                                head_decay=self.decay, k_scale=self.k_scale, **self._cutting(ctx))
         return self.o(kernels.head_norm_gate(o, None, self.eps, g, self.dtype), out_dtype=self.dtype)
