@@ -9,6 +9,7 @@ B: the values that another model may make equal or 1: value size = key size ever
    no shared expert in one layer, factors of 1, tau 1, a gla layer first, decays of 1 and near 0, one head.
 O: sizes in no kernel's favourite multiples (width 50, heads of 12, 20 and 10, 18 hidden features, 6 rotated dims of 12,
    a decay projection of rank 5): every vectorized form steps aside for its plain one, in bfloat16 too.
+G: layers of one type only, the one that keeps no pages: requests have states and lengths, and no cache to read.
 R: real-looking head sizes (64 and 128, states of 128 by 256) with few layers and pages of 64, for the matrix-core
    kernels, and key heads of more than 128 channels for the state's widest form.
 
@@ -83,6 +84,11 @@ MODELS = {
                               _moe(18, 4, 2, shared=10)),
                     _gla(3, 10, 14, 4.0, _moe(18, 3, 2))]},
         seed=23, linear_std=0.1, norm_std=0.1, page_size=8, decay_rank=5),
+    "G": dict(
+        config={"architecture": "Lilalorn", "vocab": 150, "width": 48, "norm": {"eps": 1e-5}, "residual_mult": 0.9,
+                "logit_scale": 2.0, "layers": [_gla(2, 8, 16, 2.0, None), _gla(3, 16, 8, 32.0, _moe(16, 3, 2, shared=8)),
+                                               dict(_gla(2, 8, 16, 2.0, None), weights_of=0)]},
+        seed=25, linear_std=0.15, norm_std=0.1, page_size=8, decay_rank=4),
     "R": dict(
         config={"architecture": "Lilalorn", "vocab": 409, "width": 512, "norm": {"eps": 1e-6}, "residual_mult": 0.5,
                 "logit_scale": 0.25, "layers": [

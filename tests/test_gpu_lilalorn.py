@@ -316,7 +316,8 @@ def test_a_factor_on_the_branch_that_a_norm_adds():
 
 
 # ---- whole models ----------------------------------------------------------------------------------------------
-LENGTHS = {"A": [1, 2, 12, 13, 33, 77, 130], "B": [3, 9, 10, 18, 64, 101], "O": [1, 7, 8, 40, 75], "R": [5, 101, 330, 64, 301]}
+LENGTHS = {"A": [1, 2, 12, 13, 33, 77, 130], "B": [3, 9, 10, 18, 64, 101], "O": [1, 7, 8, 40, 75], "G": [2, 1, 30, 140],
+           "R": [5, 101, 330, 64, 301]}
 
 
 def _requests(name):
@@ -475,6 +476,13 @@ def test_greedy_generation_through_the_engine(dtype, dirs):
     eng = Engine(EngineConfig(weight_path=dirs(name), page_size=16, num_pages=24, max_num_seqs=3, prefill_chunk_size=16,
                               max_model_len=128, seed=1), dtype)
     outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=24, ignore_eos=True))
+    if dtype == "f32":        # a model without pages, the engine planning its own (token counts alone)
+        g_eng = Engine(EngineConfig(weight_path=dirs("G"), page_size=8, max_num_seqs=2, prefill_chunk_size=16, max_model_len=64,
+                                    seed=1), dtype)
+        g_prompts = [[5, 9, 77, 3], list(range(40, 75))]
+        g_outs = g_eng.generate(g_prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True))
+        g_plain = plain.PlainLilalorn(dirs("G"), torch.float64)
+        assert [o.token_ids for o in g_outs] == [g_plain.greedy(p, 10) for p in g_prompts]
     pm = plain.PlainLilalorn(dirs(name), torch.float64)
     for p, o in zip(prompts, outs):
         assert o.prompt_length == len(p) and o.decoded_length == 24

@@ -13,8 +13,9 @@
 //
 // `linear_scan_kernel`: one workgroup per (item, head, 64 value columns) walks the item's tokens in order,
 // from a state it is told to start from, and may leave the new state somewhere.  Lane l owns value column l
-// of the tile, wave w the key channels w, w + 4, ..; a thread keeps its RPT state elements in registers for
-// the whole walk.  A token costs one barrier: q, k and the decay of the next token are fetched while this
+// of the tile, wave w the key channels w RPT .. (w + 1) RPT - 1 (read from LDS four at a time; channels past
+// the head's are zeros there, so the inner loop has no bounds); a thread keeps its RPT state elements in
+// registers for the whole walk.  A token costs one barrier: q, k and the decay of the next token are fetched while this
 // one is worked on.  An item is a request's tokens of this step (from the state in its slot, back into it:
 // steps of single tokens and short portions; what a token gets then does not depend on how the prompt was
 // cut, bit for bit), or one chunk of a long portion:
@@ -52,7 +53,7 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
     float* __restrict__ state_out, long long out_stride, const long long* __restrict__ out_idx,
     const int* __restrict__ first, const int* __restrict__ last, float* __restrict__ out, float* __restrict__ decay_out,
     int H, int dk, int dv, float q_scale, float k_scale) {
-  __shared__ float qs[2][kScanWaves * 64], ks[2][kScanWaves * 64], as[2][kScanWaves * 64];
+  __shared__ __attribute__((aligned(16))) float qs[2][kScanWaves * 64], ks[2][kScanWaves * 64], as[2][kScanWaves * 64];
   __shared__ float part[2][kScanWaves][kScanCols];
   const int b = blockIdx.x, h = blockIdx.y, j = blockIdx.z * kScanCols + (threadIdx.x & 63);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -64,14 +65,14 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
   float s[RPT];
 #pragma unroll
   for (int r = 0; r < RPT; ++r) {
-    const int i = wave + kScanWaves * r;
+    const int i = wave * RPT + r;
     s[r] = (from >= 0 && col && i < dk) ? S[(size_t)i * dv + j] : 0.f;
   }
   float all_decays = 1.f;               // of channel c, over the item's tokens
   const int c = threadIdx.x;            // the channel this thread fetches for the workgroup
   const float hd = head_decay ? head_decay[h] : 0.f;
   const float zb = (z_bias && c < dk) ? z_bias[h * dk + c] : 0.f;
-  auto fetch = [&](int t, float& fq, float& fk, float& fa) {
+  auto fetch = [&](int t, float& fq, float& fk, float& fa) {      // (channels past the head's stay zero)
     if (c < dk) {
       fq = to_float(q[(size_t)t * q_stride + h * dk + c]) * q_scale;
       fk = to_float(k[(size_t)t * k_stride + h * dk + c]) * k_scale;
@@ -80,28 +81,38 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
   };
   float fq = 0.f, fk = 0.f, fa = 0.f;
   fetch(t0, fq, fk, fa);
-  if (c < dk) {
-    qs[0][c] = fq;
-    ks[0][c] = fk;
-    as[0][c] = fa;
-  }
+  // the token's value is asked for a token ahead as well: no step of the walk waits for memory
+  float v_next = col ? to_float(v[(size_t)t0 * v_stride + h * dv + j]) : 0.f;
+  qs[0][c] = fq;
+  ks[0][c] = fk;
+  as[0][c] = fa;
   __syncthreads();
   for (int t = t0; t < t1; ++t) {
     const int cur = (t - t0) & 1;
     all_decays *= fa;
-    if (t + 1 < t1) fetch(t + 1, fq, fk, fa);
-    const float vj = col ? to_float(v[(size_t)t * v_stride + h * dv + j]) : 0.f;
+    const float vj = v_next;
+    if (t + 1 < t1) {
+      fetch(t + 1, fq, fk, fa);
+      if (col) v_next = to_float(v[(size_t)(t + 1) * v_stride + h * dv + j]);
+    }
     float acc = 0.f;
+    const float4* a4 = reinterpret_cast<const float4*>(&as[cur][wave * RPT]);
+    const float4* k4 = reinterpret_cast<const float4*>(&ks[cur][wave * RPT]);
+    const float4* q4 = reinterpret_cast<const float4*>(&qs[cur][wave * RPT]);
 #pragma unroll
-    for (int r = 0; r < RPT; ++r) {
-      const int i = wave + kScanWaves * r;
-      if (i < dk) {
-        s[r] = fmaf(as[cur][i], s[r], ks[cur][i] * vj);
-        acc = fmaf(s[r], qs[cur][i], acc);
-      }
+    for (int r = 0; r < RPT; r += 4) {
+      const float4 av = a4[r / 4], kv = k4[r / 4], qv = q4[r / 4];
+      s[r] = fmaf(av.x, s[r], kv.x * vj);
+      s[r + 1] = fmaf(av.y, s[r + 1], kv.y * vj);
+      s[r + 2] = fmaf(av.z, s[r + 2], kv.z * vj);
+      s[r + 3] = fmaf(av.w, s[r + 3], kv.w * vj);
+      acc = fmaf(s[r], qv.x, acc);
+      acc = fmaf(s[r + 1], qv.y, acc);
+      acc = fmaf(s[r + 2], qv.z, acc);
+      acc = fmaf(s[r + 3], qv.w, acc);
     }
     if (out) part[cur][wave][lane] = acc;
-    if (t + 1 < t1 && c < dk) {
+    if (t + 1 < t1) {
       qs[cur ^ 1][c] = fq;
       ks[cur ^ 1][c] = fk;
       as[cur ^ 1][c] = fa;
@@ -114,7 +125,7 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
     float* D = state_out + (size_t)to * out_stride + (size_t)h * dk * dv;
 #pragma unroll
     for (int r = 0; r < RPT; ++r) {
-      const int i = wave + kScanWaves * r;
+      const int i = wave * RPT + r;
       if (col && i < dk) D[(size_t)i * dv + j] = s[r];
     }
   }

@@ -85,8 +85,8 @@ def plan_pages(groups: Sequence[Tuple[int, int]], page: int, max_num_seqs: int, 
             pages = min(pages, -(-min(tokens, window - 1 + portion) // page) + 1)
         could.append(max_num_seqs * pages)
         size.append(max(1, per_token * page))
-    if not could:
-        return [1]
+    if not could:                # no layer keeps pages: the one group there is counts tokens and holds no memory
+        return [max(1, max_num_seqs * -(-max_model_len // page))]
     need = sum(c * b for c, b in zip(could, size))
     if need <= budget_bytes:
         return [max(1, c) for c in could]

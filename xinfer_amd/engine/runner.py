@@ -165,8 +165,8 @@ class ModelRunner:
         if len(num_pages) != max(1, len(needs)):
             raise ValueError(f"{len(num_pages)} page counts for {len(needs)} cache groups")
         groups = [CacheGroup(self.page_size, int(n), g.window) for g, n in zip(needs, num_pages)]
-        if not groups:                  # a model without paged layers still has state slots
-            groups = [CacheGroup(self.page_size, 0, 0)]
+        if not groups:                  # a model without paged layers still has state slots, and its requests lengths:
+            groups = [CacheGroup(self.page_size, int(num_pages[0]), 0)]     # a group that counts tokens and holds no memory
         self.cache = PagedCacheManager(groups, self.max_requests)
         self.layer_caches: Dict[int, LayerCache] = {}
         for layer, kv in model.kv_needs.items():
