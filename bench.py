@@ -268,11 +268,11 @@ def design_compare(spec: str, layers, steps: int, warmup: int, batch: int, conte
         par = {"type": "parallel", "mlp": moe, "mixer": {
             "left": dict(heads=z["heads"], kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["vdim"], scale=z["dim"] ** -0.5,
                          rot=dict(dims=z["dim"], base=500000.0, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192))),
-            "right": dict(heads=sh, dim=z["dim"], vdim=2 * z["dim"], decay=[1.0 - 2.0 ** -(5 + h % 6) for h in range(sh)]),
-            "left_scale": 0.6, "right_scale": 0.5}}
-        gla = {"type": "gla", "mlp": moe, "mixer": dict(heads=sh, dim=z["dim"], vdim=2 * z["dim"], tau=16.0)}
+            "right": dict(heads=sh, dim=z["dim"], vdim=2 * z["dim"], decay=[0.95 + 0.049 * h / max(1, sh - 1) for h in range(sh)]),
+            "left_scale": 0.75, "right_scale": 0.4}}
+        gla = {"type": "gla", "mlp": moe, "mixer": dict(heads=sh, dim=z["dim"], vdim=2 * z["dim"], tau=8.0)}
         lilalorn = {"architecture": "Lilalorn", "vocab": DESIGN_VOCAB, "width": z["width"], "norm": {"eps": 1e-6},
-                    "residual_mult": 0.7, "logit_scale": 0.5, "max_positions": 2 * context,
+                    "residual_mult": 0.8, "logit_scale": 0.25, "max_positions": 2 * context,
                     "layers": [par if i % 2 == 0 else gla for i in range(layers)]}
         return {"lilalorn": lilalorn, "mufenex": mufenex}
 

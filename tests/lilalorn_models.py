@@ -76,7 +76,7 @@ MODELS = {
                     _parallel(_left(2, 2, 32, 32, 0.18, rot_dims=32, base=1000.0), _right(2, 8, 8, [0.05, 1.0]), 1.0, 1.0,
                               _moe(16, 2, 2, shared=8)),
                     dict(_B1, weights_of=1)]},
-        seed=22, linear_std=0.12, norm_std=0.2, page_size=8, decay_rank=16),
+        seed=22, linear_std=0.12, norm_std=0.2, page_size=8, decay_rank=12),
     "O": dict(
         config={"architecture": "Lilalorn", "vocab": 131, "width": 50, "norm": {"eps": 1e-5}, "residual_mult": 0.8,
                 "logit_scale": 1.5, "layers": [
@@ -94,9 +94,9 @@ MODELS = {
                 "logit_scale": 0.25, "layers": [
                     _parallel(_left(8, 2, 64, 128, 0.125, rot_dims=64, base=500000.0, scaling=(8.0, 1.0, 4.0, 8192)),
                               _right(4, 64, 128, [0.97, 0.99, 0.995, 0.999]), 0.7, 0.5, _moe(128, 6, 2, shared=256)),
-                    _gla(2, 128, 256, 16.0, _moe(128, 6, 2, shared=256)),
-                    _gla(1, 192, 64, 16.0, None)]},
-        seed=24, linear_std=0.04, norm_std=0.1, page_size=64, decay_rank=16),
+                    _gla(2, 128, 256, 12.0, _moe(128, 6, 2, shared=256)),
+                    _gla(1, 192, 64, 20.0, None)]},
+        seed=24, linear_std=0.04, norm_std=0.1, page_size=64, decay_rank=24),
 }
 
 

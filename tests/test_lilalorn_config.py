@@ -52,7 +52,7 @@ def test_the_decay_rank_is_the_checkpoints(tmp_path):
         spec = fam.spec(cfg, ShapedNames(store))
     finally:
         store.close()
-    assert spec.layers[1].mixer["decay_rank"] == 5 and fam.spec(cfg).layers[1].mixer["decay_rank"] == 16
+    assert spec.layers[1].mixer["decay_rank"] == 5 and fam.spec(cfg).layers[1].mixer["decay_rank"] == 32
 
 
 @pytest.mark.parametrize("change,message", [

@@ -292,7 +292,8 @@ def test_pages_are_planned_group_by_group():
     half = plan_pages([full, windowed], page, seqs, length, portion, need // 2)
     assert half == [512, 14]
     assert plan_pages([full, windowed], page, seqs, length, portion, 1) == [1, 1]
-    assert plan_pages([], page, seqs, length, portion, 1 << 40) == [1]
+    # no layer keeps pages: the one group counts the requests' tokens and holds no memory
+    assert plan_pages([], page, seqs, length, portion, 1) == [seqs * (length // page)]
     # what was planned is what the scheduler needs for max_num_seqs requests of the full length:
     # all are admitted together and nothing is ever preempted
     cm = PagedCacheManager([CacheGroup(page, got[0]), CacheGroup(page, got[1], window=24)], max_requests=seqs)

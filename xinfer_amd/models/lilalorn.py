@@ -38,7 +38,7 @@ from ..config.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
 from .registry import ModelFamily, register_architecture
 
 DEFAULT_POSITIONS = 1 << 16       # config.json names no longest sequence: what the engine plans its tables for
-DEFAULT_DECAY_RANK = 16           # of random weights; a checkpoint's own is read from its tensor
+DEFAULT_DECAY_RANK = 32           # of random weights; a checkpoint's own is read from its tensor
 
 
 def _opt(raw: Optional[Dict[str, Any]], key: str, typ, where: str):
